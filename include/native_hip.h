@@ -1,0 +1,168 @@
+/* native-hip: C ABI of the MI355X (gfx950) matrix executor for llama-rust's
+ * GGUF block-quantized matrix products.
+ *
+ * This is the boundary a Rust `native-hip` crate binds (one `extern "C"` block,
+ * no other FFI), and the only way host code reaches the HIP kernels.  Every
+ * entry point names the reference interface it stands in for; paths are
+ * relative to the reference checkout.
+ *
+ * Conventions
+ *   - Plain pointers and sizes only.  `*_len` arguments are ELEMENT counts of
+ *     the buffer they follow (f32 elements, or bytes for packed weights).
+ *   - Return value: LNH_OK (0) or an lnh_status error code.  The message of the
+ *     most recent failure on an executor is lnh_last_error(exec); for calls
+ *     without an executor (lnh_create, lnq_*) it is lnh_thread_error() /
+ *     lnq_last_error(), both thread-local.  Strings stay valid until the next
+ *     call on the same executor / thread.
+ *   - Validation happens before any device work and never touches `y`.
+ *     After any error the executor remains usable.
+ *   - There is no CPU fallback: a missing device or a failed launch is an error.
+ *   - An executor and its matrices are confined to one host thread at a time
+ *     (the reference takes `&mut self` on every operation).
+ *   - Products are token-major: x[t*cols + c], y[t*rows + r],
+ *     y[t, r] = sum_c W[r, c] * x[t, c], f32 activations, f32 accumulation.
+ */
+#ifndef NATIVE_HIP_H
+#define NATIVE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct lnh_exec lnh_exec;     /* stands in for CudaGemv   (native-cuda/src/gpu.rs:132-141) */
+typedef struct lnh_matrix lnh_matrix; /* stands in for CudaMatrix (native-cuda/src/gpu.rs:125-130) */
+
+typedef enum lnh_status {
+    LNH_OK = 0,
+    LNH_ERR_INVALID = 1,     /* shape / length / argument validation failed; nothing was launched */
+    LNH_ERR_DEVICE = 2,      /* a HIP runtime call or kernel failed */
+    LNH_ERR_OOM = 3,         /* device allocation failed (after the scratch pool was released and retried) */
+    LNH_ERR_FOREIGN = 4,     /* matrix belongs to a different executor */
+    LNH_ERR_UNSUPPORTED = 5  /* dtype outside F32, F16, Q4_0, Q4_K, Q5_0, Q5_1, Q6_K, Q8_0 */
+} lnh_status;
+
+/* ggml type ids (langtax/src/gguf.rs:245-258); the Rust shim maps GemmKind to these. */
+enum {
+    LNH_TYPE_F32 = 0,
+    LNH_TYPE_F16 = 1,
+    LNH_TYPE_Q4_0 = 2,
+    LNH_TYPE_Q5_0 = 6,
+    LNH_TYPE_Q5_1 = 7,
+    LNH_TYPE_Q8_0 = 8,
+    LNH_TYPE_Q4_K = 12,
+    LNH_TYPE_Q6_K = 14
+};
+
+/* ------------------------------------------------------------------ executor */
+
+/* CudaGemv::new(device_ordinal)            native-cuda/src/gpu.rs:148-161 */
+int lnh_create(int device_ordinal, lnh_exec **out);
+void lnh_destroy(lnh_exec *exec);
+/* CudaGemv::memory_info -> (free, total)   native-cuda/src/gpu.rs:164-175 */
+int lnh_memory_info(lnh_exec *exec, size_t *free_bytes, size_t *total_bytes);
+/* Err(String) of the last failed call on this executor ("" if none). */
+const char *lnh_last_error(const lnh_exec *exec);
+/* Message of the last failed lnh_create / host-only helper on this thread. */
+const char *lnh_thread_error(void);
+
+/* ------------------------------------------------------------------ resident matrices */
+
+/* CudaGemv::upload(rows, cols, &[f32])     native-cuda/src/gpu.rs:264-277
+ * Same checks and messages as Shape::checked (native-cuda/src/lib.rs:19-34). */
+int lnh_upload_f32(lnh_exec *exec, size_t rows, size_t cols, const float *weights, size_t weights_len,
+                   lnh_matrix **out);
+/* Packed residency: takes the GGUF bytes of a rows x cols tensor as they lie in
+ * the file and keeps them packed in HBM.  Replaces the host-side expansion to
+ * F32 at langtax/src/quant.rs:6746-6755 followed by upload (native_gpu.rs:190-194).
+ * `nbytes` must equal rows * row_bytes(type, cols); cols must be a whole number
+ * of blocks (32 for Q4_0/Q5_0/Q5_1/Q8_0, 256 for Q4_K/Q6_K). */
+int lnh_upload_packed(lnh_exec *exec, uint32_t ggml_type, size_t rows, size_t cols, const uint8_t *bytes,
+                      size_t nbytes, lnh_matrix **out);
+/* Same, from bytes that already sit in device memory of this executor's GPU. */
+int lnh_upload_packed_device(lnh_exec *exec, uint32_t ggml_type, size_t rows, size_t cols,
+                             const void *device_bytes, size_t nbytes, lnh_matrix **out);
+/* Drop of a CudaMatrix.  Safe after its executor was destroyed. */
+void lnh_matrix_free(lnh_matrix *matrix);
+int lnh_matrix_info(const lnh_matrix *matrix, uint32_t *ggml_type, size_t *rows, size_t *cols,
+                    size_t *device_bytes);
+
+/* ------------------------------------------------------------------ products (host buffers) */
+
+/* CudaGemv::gemv_resident(matrix, input, output)          native-cuda/src/gpu.rs:280-335 */
+int lnh_gemv(lnh_exec *exec, const lnh_matrix *matrix, const float *x, size_t x_len, float *y, size_t y_len);
+/* CudaGemv::gemm_resident(matrix, tokens, input, output)  native-cuda/src/gpu.rs:351-417
+ * (tokens == 1 runs the GEMV kernel; native_gpu::matmul always calls this one). */
+int lnh_gemm(lnh_exec *exec, const lnh_matrix *matrix, size_t tokens, const float *x, size_t x_len, float *y,
+             size_t y_len);
+/* CudaGemv::gemv(weights, input, output): upload + product native-cuda/src/gpu.rs:339-347 */
+int lnh_gemv_once(lnh_exec *exec, const float *weights, size_t weights_len, const float *x, size_t x_len,
+                  float *y, size_t y_len);
+/* Expert-grouped GEMM: group g multiplies tokens[g] packed rows of x by mats[g].
+ * Stands in for the per-expert loop of three gemm calls at
+ * langtax/src/decode.rs:10035-10058 / 10148-10261 (one call per projection).
+ * x holds the groups' token rows back to back (sum_g tokens[g]*cols[g] floats),
+ * y likewise (sum_g tokens[g]*rows[g]).  Groups with tokens[g] == 0 are skipped. */
+int lnh_gemm_grouped(lnh_exec *exec, size_t n_groups, const lnh_matrix *const *mats, const size_t *tokens,
+                     const float *x, size_t x_len, float *y, size_t y_len);
+
+/* ------------------------------------------------------------------ products (device buffers) */
+
+/* The same products with x and y already in this GPU's memory, enqueued on
+ * `stream` (a hipStream_t; NULL = the executor's own stream) without any host
+ * synchronisation.  No counterpart in the reference, whose every call copies
+ * through the host (native-cuda/src/gpu.rs:301-303, 332-334). */
+int lnh_gemm_device(lnh_exec *exec, const lnh_matrix *matrix, size_t tokens, const float *device_x,
+                    float *device_y, void *stream);
+int lnh_gemm_grouped_device(lnh_exec *exec, size_t n_groups, const lnh_matrix *const *mats,
+                            const size_t *tokens, const float *device_x, float *device_y, void *stream);
+/* Block the host until everything enqueued on the executor's own stream is done. */
+int lnh_synchronize(lnh_exec *exec);
+
+/* ------------------------------------------------------------------ host-only helpers */
+
+/* Shape::checked(rows, cols, weights, input)   native-cuda/src/lib.rs:19-34 */
+int lnh_shape_checked(size_t rows, size_t cols, size_t weights_len, size_t input_len, uint32_t *rows_out,
+                      uint32_t *cols_out);
+/* validate(actual, expected)                   native-cuda/src/lib.rs:37-53
+ * Returns LNH_OK when every |a-e| <= 1e-4 + 1e-4|e| with both finite. */
+int lnh_validate(const float *actual, size_t actual_len, const double *expected, size_t expected_len);
+/* Packed bytes of one row, 0 if cols is not a whole number of blocks or the type is unknown
+ * (langtax/src/quant.rs:4210-4218, 4254-4284, 5647-5682). */
+size_t lnh_row_bytes(uint32_t ggml_type, size_t cols);
+
+/* ------------------------------------------------------------------ dispatch + residency
+ * The layer above the executor: the twin of langtax/src/native_gpu.rs plus the
+ * validation of quant::native_matmul (langtax/src/quant.rs:6683-6758), i.e. what
+ * gemv_<t>_f32 / gemm_<t>_f32 (quant.rs:6144-6293, 6366-6478, 6891-7199) run
+ * when the GPU backend is compiled in.  One executor and one residency cache
+ * per host thread; identity of a weight is its dtype, shape and ALL its bytes. */
+
+/* gemv_<t>_f32(n_cols, w, x, y):  n_rows = y_len */
+int lnq_gemv(uint32_t ggml_type, size_t n_cols, const uint8_t *w, size_t w_len, const float *x, size_t x_len,
+             float *y, size_t y_len);
+/* gemm_<t>_f32(n_cols, n_tokens, w, x, y):  n_rows = y_len / n_tokens */
+int lnq_gemm(uint32_t ggml_type, size_t n_cols, size_t n_tokens, const uint8_t *w, size_t w_len,
+             const float *x, size_t x_len, float *y, size_t y_len);
+/* The per-expert products of one MoE projection in one call; part g is the
+ * byte slice of expert g (langtax/src/decode.rs:9853-9913).  All parts share
+ * dtype, n_cols and n_rows. */
+int lnq_gemm_grouped(uint32_t ggml_type, size_t n_cols, size_t n_rows, size_t n_groups,
+                     const uint8_t *const *parts, size_t part_len, const size_t *tokens, const float *x,
+                     size_t x_len, float *y, size_t y_len);
+const char *lnq_last_error(void);
+/* Residency policy, exposed for host tests (native_gpu.rs:20-43, 217-360). */
+int lnq_parse_cache_bytes(const char *value_or_null, int *is_auto, size_t *bytes);
+size_t lnq_automatic_cache_bytes(size_t free_bytes, size_t total_bytes);
+int lnq_admission_requires_eviction(size_t used, size_t incoming, size_t limit);
+/* Counters of this thread's cache; any pointer may be NULL. */
+void lnq_cache_stats(size_t *entries, size_t *bytes, size_t *limit, size_t *hits, size_t *misses);
+/* Drop this thread's executor and cache (the next call re-reads LLAMA_HIP_CACHE_BYTES). */
+void lnq_reset(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,446 @@
+// C ABI of the executor (include/native_hip.h): device context, resident
+// matrices, scratch reuse and the validation rules of the reference's
+// CudaGemv / CudaMatrix / Shape / validate
+// (native-cuda/src/gpu.rs:125-418, native-cuda/src/lib.rs:8-53).
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "../../include/native_hip.h"
+#include "kernels.h"
+
+namespace {
+
+struct Ctx {
+    int device;
+    uint64_t id;
+};
+
+std::atomic<uint64_t> g_next_ctx{1};
+thread_local std::string t_error;
+
+}  // namespace
+
+struct lnh_matrix {
+    std::shared_ptr<Ctx> ctx;
+    void *dev = nullptr;
+    size_t dev_bytes = 0;
+    nh::MatView view{};
+};
+
+struct lnh_exec {
+    std::shared_ptr<Ctx> ctx;
+    hipStream_t stream = nullptr;
+    float *d_in = nullptr, *d_out = nullptr;  // device scratch, grow-only
+    size_t in_cap = 0, out_cap = 0;           // capacities in floats
+    std::string err;
+};
+
+namespace {
+
+int fail(lnh_exec *e, int code, const std::string &msg) {
+    if (e) e->err = msg;
+    t_error = msg;
+    return code;
+}
+
+int hip_fail(lnh_exec *e, hipError_t h, const char *what) {
+    (void)hipGetLastError();  // clear the sticky error so the executor stays usable
+    int code = h == hipErrorOutOfMemory ? LNH_ERR_OOM : LNH_ERR_DEVICE;
+    return fail(e, code, std::string(what) + ": " + hipGetErrorString(h));
+}
+
+bool mul_overflows(size_t a, size_t b, size_t *out) {
+    if (a != 0 && b > SIZE_MAX / a) return true;
+    *out = a * b;
+    return false;
+}
+
+// native-cuda/src/lib.rs:19-34, message for message.
+const char *shape_checked(size_t rows, size_t cols, size_t weights, size_t input, uint32_t *r32, uint32_t *c32) {
+    if (rows == 0 || cols == 0) return "GEMV dimensions must be positive";
+    size_t elements;
+    if (mul_overflows(rows, cols, &elements)) return "GEMV shape overflow";
+    if (elements > UINT32_MAX) return "GEMV matrix exceeds u32 indexing";
+    if (weights != elements || input != cols) return "GEMV buffer lengths do not match shape";
+    if (rows > UINT32_MAX) return "GEMV rows exceed u32";
+    if (cols > UINT32_MAX) return "GEMV columns exceed u32";
+    if (r32) *r32 = (uint32_t)rows;
+    if (c32) *c32 = (uint32_t)cols;
+    return nullptr;
+}
+
+// Device scratch that recurring shapes reuse across layers and tokens
+// (native-cuda/src/gpu.rs:143-262).  Grow-only; an out-of-memory on growth
+// releases both buffers and retries once (gpu.rs:198-210).
+int ensure_scratch(lnh_exec *e, size_t in_floats, size_t out_floats) {
+    auto grow = [&](float *&buf, size_t &cap, size_t want) -> hipError_t {
+        if (want <= cap) return hipSuccess;
+        if (buf) {
+            (void)hipFree(buf);
+            buf = nullptr;
+            cap = 0;
+        }
+        size_t n = want < 4096 ? 4096 : want;
+        hipError_t h = hipMalloc(reinterpret_cast<void **>(&buf), n * sizeof(float));
+        if (h == hipSuccess) cap = n;
+        return h;
+    };
+    for (int attempt = 0; attempt < 2; attempt++) {
+        hipError_t h = grow(e->d_in, e->in_cap, in_floats);
+        if (h == hipSuccess) h = grow(e->d_out, e->out_cap, out_floats);
+        if (h == hipSuccess) return LNH_OK;
+        (void)hipGetLastError();
+        if (h != hipErrorOutOfMemory || attempt == 1) return hip_fail(e, h, "HIP scratch allocation");
+        if (e->d_in) (void)hipFree(e->d_in);
+        if (e->d_out) (void)hipFree(e->d_out);
+        e->d_in = e->d_out = nullptr;
+        e->in_cap = e->out_cap = 0;
+    }
+    return LNH_ERR_OOM;
+}
+
+int make_matrix(lnh_exec *e, uint32_t type, size_t rows, size_t cols, const void *src, bool src_on_device,
+                size_t nbytes, lnh_matrix **out) {
+    nh::PlaneSpec ps = nh::plane_spec(type, rows, cols);
+    hipError_t h = hipSetDevice(e->ctx->device);
+    if (h != hipSuccess) return hip_fail(e, h, "hipSetDevice");
+    void *dev = nullptr;
+    h = hipMalloc(&dev, ps.total);
+    if (h != hipSuccess) return hip_fail(e, h, "HIP matrix allocation");
+    void *staging = nullptr;
+    const void *src_dev = src;
+    if (!src_on_device) {
+        h = hipMalloc(&staging, nbytes ? nbytes : 1);
+        if (h != hipSuccess) {
+            (void)hipFree(dev);
+            return hip_fail(e, h, "HIP upload staging allocation");
+        }
+        h = hipMemcpyAsync(staging, src, nbytes, hipMemcpyHostToDevice, e->stream);
+        src_dev = staging;
+    }
+    auto m = std::make_unique<lnh_matrix>();
+    m->ctx = e->ctx;
+    m->dev = dev;
+    m->dev_bytes = ps.total;
+    uint8_t *base = static_cast<uint8_t *>(dev);
+    m->view.p0 = base + ps.offset[0];
+    m->view.p1 = base + ps.offset[1];
+    m->view.p2 = base + ps.offset[2];
+    m->view.p3 = base + ps.offset[3];
+    m->view.s0 = (uint32_t)ps.stride[0];
+    m->view.s1 = (uint32_t)ps.stride[1];
+    m->view.s2 = (uint32_t)ps.stride[2];
+    m->view.s3 = (uint32_t)ps.stride[3];
+    m->view.type = type;
+    m->view.rows = (uint32_t)rows;
+    m->view.cols = (uint32_t)cols;
+    m->view.nb = (uint32_t)(cols / nh::block_elems(type));
+    if (h == hipSuccess) h = nh::launch_repack(e->stream, m->view, src_dev);
+    hipError_t hs = hipStreamSynchronize(e->stream);
+    if (h == hipSuccess) h = hs;
+    if (staging) (void)hipFree(staging);
+    if (h != hipSuccess) {
+        (void)hipFree(dev);
+        return hip_fail(e, h, "HIP matrix upload");
+    }
+    *out = m.release();
+    return LNH_OK;
+}
+
+int check_packed_shape(lnh_exec *e, uint32_t type, size_t rows, size_t cols, size_t nbytes) {
+    if (!nh::type_supported(type)) return fail(e, LNH_ERR_UNSUPPORTED, "unsupported GGUF dtype " + std::to_string(type));
+    if (rows == 0 || cols == 0) return fail(e, LNH_ERR_INVALID, "GEMV dimensions must be positive");
+    size_t qk = nh::block_elems(type);
+    if (cols % qk != 0)
+        return fail(e, LNH_ERR_INVALID, "n_cols " + std::to_string(cols) + " is not a multiple of " + std::to_string(qk));
+    if (rows > UINT32_MAX) return fail(e, LNH_ERR_INVALID, "GEMV rows exceed u32");
+    if (cols > UINT32_MAX) return fail(e, LNH_ERR_INVALID, "GEMV columns exceed u32");
+    size_t rb = nh::gguf_row_bytes(type, cols), total;
+    if (rb == 0 || mul_overflows(rb, rows, &total)) return fail(e, LNH_ERR_INVALID, "GEMV shape overflow");
+    if (nbytes != total) return fail(e, LNH_ERR_INVALID, "GEMV buffer lengths do not match shape");
+    // plane strides are kept in 32 bits
+    if (nh::plane_spec(type, 1, cols).stride[0] > UINT32_MAX) return fail(e, LNH_ERR_INVALID, "GEMV columns exceed u32");
+    return LNH_OK;
+}
+
+// Shared checks of gemm_resident (native-cuda/src/gpu.rs:358-371).
+int check_gemm(lnh_exec *e, const lnh_matrix *m, size_t tokens, bool have_lens, size_t x_len, size_t y_len,
+               size_t *inputs, size_t *outputs) {
+    if (!e) return LNH_ERR_INVALID;
+    if (!m) return fail(e, LNH_ERR_INVALID, "HIP matrix is null");
+    if (m->ctx.get() != e->ctx.get()) return fail(e, LNH_ERR_FOREIGN, "HIP matrix belongs to a different executor");
+    if (mul_overflows(tokens, m->view.cols, inputs)) return fail(e, LNH_ERR_INVALID, "HIP GEMM input shape overflow");
+    if (mul_overflows(tokens, m->view.rows, outputs)) return fail(e, LNH_ERR_INVALID, "HIP GEMM output shape overflow");
+    if (tokens == 0 || (have_lens && (x_len != *inputs || y_len != *outputs)))
+        return fail(e, LNH_ERR_INVALID, "HIP GEMM buffer lengths do not match shape");
+    if (*outputs > UINT32_MAX) return fail(e, LNH_ERR_INVALID, "HIP GEMM launch exceeds u32");
+    if (*inputs > UINT32_MAX) return fail(e, LNH_ERR_INVALID, "HIP GEMM input exceeds u32");
+    return LNH_OK;
+}
+
+// H2D x, kernel(s), blocking D2H y (native-cuda/src/gpu.rs:301-303, 332-334).
+int run_host(lnh_exec *e, size_t n_groups, const lnh_matrix *const *mats, const size_t *tokens, const float *x,
+             size_t x_total, float *y, size_t y_total) {
+    hipError_t h = hipSetDevice(e->ctx->device);
+    if (h != hipSuccess) return hip_fail(e, h, "hipSetDevice");
+    int rc = ensure_scratch(e, x_total, y_total);
+    if (rc != LNH_OK) return rc;
+    h = hipMemcpyAsync(e->d_in, x, x_total * sizeof(float), hipMemcpyHostToDevice, e->stream);
+    if (h != hipSuccess) return hip_fail(e, h, "HIP input copy");
+    size_t xo = 0, yo = 0;
+    for (size_t g = 0; g < n_groups; g++) {
+        if (tokens[g] == 0) continue;
+        h = nh::launch_gemm(e->stream, mats[g]->view, (uint32_t)tokens[g], e->d_in + xo, e->d_out + yo);
+        if (h != hipSuccess) {
+            (void)hipStreamSynchronize(e->stream);
+            return hip_fail(e, h, "HIP kernel launch");
+        }
+        xo += tokens[g] * mats[g]->view.cols;
+        yo += tokens[g] * mats[g]->view.rows;
+    }
+    h = hipMemcpyAsync(y, e->d_out, y_total * sizeof(float), hipMemcpyDeviceToHost, e->stream);
+    hipError_t hs = hipStreamSynchronize(e->stream);
+    if (h == hipSuccess) h = hs;
+    if (h != hipSuccess) return hip_fail(e, h, "HIP output copy");
+    return LNH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int lnh_create(int device_ordinal, lnh_exec **out) {
+    if (!out) return fail(nullptr, LNH_ERR_INVALID, "lnh_create: out is null");
+    *out = nullptr;
+    int count = 0;
+    hipError_t h = hipGetDeviceCount(&count);
+    if (h != hipSuccess) return hip_fail(nullptr, h, "hipGetDeviceCount");
+    if (device_ordinal < 0 || device_ordinal >= count)
+        return fail(nullptr, LNH_ERR_DEVICE,
+                    "HIP device " + std::to_string(device_ordinal) + " not present (" + std::to_string(count) +
+                        " visible); no CPU fallback");
+    h = hipSetDevice(device_ordinal);
+    if (h != hipSuccess) return hip_fail(nullptr, h, "hipSetDevice");
+    hipDeviceProp_t prop;
+    h = hipGetDeviceProperties(&prop, device_ordinal);
+    if (h != hipSuccess) return hip_fail(nullptr, h, "hipGetDeviceProperties");
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(nullptr, LNH_ERR_DEVICE, std::string("kernels are built for gfx950 only, device is ") + prop.gcnArchName);
+    size_t lds = prop.sharedMemPerBlockOptin ? prop.sharedMemPerBlockOptin : prop.sharedMemPerBlock;
+    if (lds > 80 * 1024) lds = 80 * 1024;  // two workgroups per CU must fit in the 160 KB LDS
+    nh::set_device_limits(prop.multiProcessorCount, lds);
+    auto e = std::make_unique<lnh_exec>();
+    e->ctx = std::make_shared<Ctx>();
+    e->ctx->device = device_ordinal;
+    e->ctx->id = g_next_ctx.fetch_add(1);
+    h = hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking);
+    if (h != hipSuccess) return hip_fail(nullptr, h, "hipStreamCreate");
+    *out = e.release();
+    return LNH_OK;
+}
+
+void lnh_destroy(lnh_exec *e) {
+    if (!e) return;
+    (void)hipSetDevice(e->ctx->device);
+    if (e->stream) {
+        (void)hipStreamSynchronize(e->stream);
+        (void)hipStreamDestroy(e->stream);
+    }
+    if (e->d_in) (void)hipFree(e->d_in);
+    if (e->d_out) (void)hipFree(e->d_out);
+    delete e;
+}
+
+int lnh_memory_info(lnh_exec *e, size_t *free_bytes, size_t *total_bytes) {
+    if (!e) return LNH_ERR_INVALID;
+    hipError_t h = hipSetDevice(e->ctx->device);
+    size_t f = 0, t = 0;
+    if (h == hipSuccess) h = hipMemGetInfo(&f, &t);
+    if (h != hipSuccess) return hip_fail(e, h, "hipMemGetInfo");
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+    return LNH_OK;
+}
+
+const char *lnh_last_error(const lnh_exec *e) { return e ? e->err.c_str() : ""; }
+const char *lnh_thread_error(void) { return t_error.c_str(); }
+
+int lnh_upload_f32(lnh_exec *e, size_t rows, size_t cols, const float *weights, size_t weights_len, lnh_matrix **out) {
+    if (!e || !out) return LNH_ERR_INVALID;
+    *out = nullptr;
+    if (const char *msg = shape_checked(rows, cols, weights_len, cols, nullptr, nullptr))
+        return fail(e, LNH_ERR_INVALID, msg);
+    if (!weights) return fail(e, LNH_ERR_INVALID, "weights pointer is null");
+    return make_matrix(e, nh::T_F32, rows, cols, weights, false, weights_len * sizeof(float), out);
+}
+
+int lnh_upload_packed(lnh_exec *e, uint32_t type, size_t rows, size_t cols, const uint8_t *bytes, size_t nbytes,
+                      lnh_matrix **out) {
+    if (!e || !out) return LNH_ERR_INVALID;
+    *out = nullptr;
+    int rc = check_packed_shape(e, type, rows, cols, nbytes);
+    if (rc != LNH_OK) return rc;
+    if (!bytes) return fail(e, LNH_ERR_INVALID, "weights pointer is null");
+    return make_matrix(e, type, rows, cols, bytes, false, nbytes, out);
+}
+
+int lnh_upload_packed_device(lnh_exec *e, uint32_t type, size_t rows, size_t cols, const void *device_bytes,
+                             size_t nbytes, lnh_matrix **out) {
+    if (!e || !out) return LNH_ERR_INVALID;
+    *out = nullptr;
+    int rc = check_packed_shape(e, type, rows, cols, nbytes);
+    if (rc != LNH_OK) return rc;
+    if (!device_bytes) return fail(e, LNH_ERR_INVALID, "weights pointer is null");
+    return make_matrix(e, type, rows, cols, device_bytes, true, nbytes, out);
+}
+
+void lnh_matrix_free(lnh_matrix *m) {
+    if (!m) return;
+    (void)hipSetDevice(m->ctx->device);
+    if (m->dev) (void)hipFree(m->dev);
+    delete m;
+}
+
+int lnh_matrix_info(const lnh_matrix *m, uint32_t *type, size_t *rows, size_t *cols, size_t *device_bytes) {
+    if (!m) return LNH_ERR_INVALID;
+    if (type) *type = m->view.type;
+    if (rows) *rows = m->view.rows;
+    if (cols) *cols = m->view.cols;
+    if (device_bytes) *device_bytes = m->dev_bytes;
+    return LNH_OK;
+}
+
+int lnh_gemv(lnh_exec *e, const lnh_matrix *m, const float *x, size_t x_len, float *y, size_t y_len) {
+    if (!e) return LNH_ERR_INVALID;
+    if (!m) return fail(e, LNH_ERR_INVALID, "HIP matrix is null");
+    if (m->ctx.get() != e->ctx.get()) return fail(e, LNH_ERR_FOREIGN, "HIP matrix belongs to a different executor");
+    if (x_len != m->view.cols || y_len != m->view.rows)
+        return fail(e, LNH_ERR_INVALID, "HIP GEMV vector lengths do not match resident matrix");
+    if (!x || !y) return fail(e, LNH_ERR_INVALID, "vector pointer is null");
+    size_t one = 1;
+    return run_host(e, 1, &m, &one, x, x_len, y, y_len);
+}
+
+int lnh_gemm(lnh_exec *e, const lnh_matrix *m, size_t tokens, const float *x, size_t x_len, float *y, size_t y_len) {
+    size_t inputs, outputs;
+    int rc = check_gemm(e, m, tokens, true, x_len, y_len, &inputs, &outputs);
+    if (rc != LNH_OK) return rc;
+    if (!x || !y) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    return run_host(e, 1, &m, &tokens, x, inputs, y, outputs);
+}
+
+int lnh_gemv_once(lnh_exec *e, const float *weights, size_t weights_len, const float *x, size_t x_len, float *y,
+                  size_t y_len) {
+    if (!e) return LNH_ERR_INVALID;
+    lnh_matrix *m = nullptr;
+    // upload(output.len(), input.len(), weights)
+    if (const char *msg = shape_checked(y_len, x_len, weights_len, x_len, nullptr, nullptr))
+        return fail(e, LNH_ERR_INVALID, msg);
+    int rc = lnh_upload_f32(e, y_len, x_len, weights, weights_len, &m);
+    if (rc != LNH_OK) return rc;
+    rc = lnh_gemv(e, m, x, x_len, y, y_len);
+    lnh_matrix_free(m);
+    return rc;
+}
+
+static int check_groups(lnh_exec *e, size_t n_groups, const lnh_matrix *const *mats, const size_t *tokens,
+                        size_t *x_total, size_t *y_total) {
+    if (!e) return LNH_ERR_INVALID;
+    if (n_groups != 0 && (!mats || !tokens)) return fail(e, LNH_ERR_INVALID, "group arrays are null");
+    size_t xt = 0, yt = 0;
+    for (size_t g = 0; g < n_groups; g++) {
+        if (!mats[g]) return fail(e, LNH_ERR_INVALID, "HIP matrix is null");
+        if (mats[g]->ctx.get() != e->ctx.get())
+            return fail(e, LNH_ERR_FOREIGN, "HIP matrix belongs to a different executor");
+        size_t in, outn;
+        if (mul_overflows(tokens[g], mats[g]->view.cols, &in) || mul_overflows(tokens[g], mats[g]->view.rows, &outn) ||
+            xt + in < xt || yt + outn < yt)
+            return fail(e, LNH_ERR_INVALID, "HIP GEMM input shape overflow");
+        if (in > UINT32_MAX || outn > UINT32_MAX) return fail(e, LNH_ERR_INVALID, "HIP GEMM launch exceeds u32");
+        xt += in;
+        yt += outn;
+    }
+    *x_total = xt;
+    *y_total = yt;
+    return LNH_OK;
+}
+
+int lnh_gemm_grouped(lnh_exec *e, size_t n_groups, const lnh_matrix *const *mats, const size_t *tokens, const float *x,
+                     size_t x_len, float *y, size_t y_len) {
+    size_t xt, yt;
+    int rc = check_groups(e, n_groups, mats, tokens, &xt, &yt);
+    if (rc != LNH_OK) return rc;
+    if (x_len != xt || y_len != yt) return fail(e, LNH_ERR_INVALID, "HIP GEMM buffer lengths do not match shape");
+    if (yt == 0) return LNH_OK;
+    if (!x || !y) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    return run_host(e, n_groups, mats, tokens, x, xt, y, yt);
+}
+
+int lnh_gemm_device(lnh_exec *e, const lnh_matrix *m, size_t tokens, const float *dx, float *dy, void *stream) {
+    size_t inputs, outputs;
+    int rc = check_gemm(e, m, tokens, false, 0, 0, &inputs, &outputs);
+    if (rc != LNH_OK) return rc;
+    if (!dx || !dy) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
+    hipError_t h = nh::launch_gemm(s, m->view, (uint32_t)tokens, dx, dy);
+    if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
+    return LNH_OK;
+}
+
+int lnh_gemm_grouped_device(lnh_exec *e, size_t n_groups, const lnh_matrix *const *mats, const size_t *tokens,
+                            const float *dx, float *dy, void *stream) {
+    size_t xt, yt;
+    int rc = check_groups(e, n_groups, mats, tokens, &xt, &yt);
+    if (rc != LNH_OK) return rc;
+    if (yt == 0) return LNH_OK;
+    if (!dx || !dy) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
+    size_t xo = 0, yo = 0;
+    for (size_t g = 0; g < n_groups; g++) {
+        if (tokens[g] == 0) continue;
+        hipError_t h = nh::launch_gemm(s, mats[g]->view, (uint32_t)tokens[g], dx + xo, dy + yo);
+        if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
+        xo += tokens[g] * mats[g]->view.cols;
+        yo += tokens[g] * mats[g]->view.rows;
+    }
+    return LNH_OK;
+}
+
+int lnh_synchronize(lnh_exec *e) {
+    if (!e) return LNH_ERR_INVALID;
+    hipError_t h = hipStreamSynchronize(e->stream);
+    if (h != hipSuccess) return hip_fail(e, h, "hipStreamSynchronize");
+    return LNH_OK;
+}
+
+int lnh_shape_checked(size_t rows, size_t cols, size_t weights_len, size_t input_len, uint32_t *rows_out,
+                      uint32_t *cols_out) {
+    if (const char *msg = shape_checked(rows, cols, weights_len, input_len, rows_out, cols_out))
+        return fail(nullptr, LNH_ERR_INVALID, msg);
+    return LNH_OK;
+}
+
+int lnh_validate(const float *actual, size_t actual_len, const double *expected, size_t expected_len) {
+    if (actual_len != expected_len) return fail(nullptr, LNH_ERR_INVALID, "GEMV output length mismatch");
+    for (size_t i = 0; i < actual_len; i++) {
+        double a = (double)actual[i], ex = expected[i];
+        double tol = 1e-4 + 1e-4 * std::fabs(ex);
+        if (!std::isfinite(a) || !std::isfinite(ex) || std::fabs(a - ex) > tol) {
+            char buf[160];
+            std::snprintf(buf, sizeof buf, "GEMV mismatch at row %zu: expected %.17g, got %.9g", i, ex, a);
+            return fail(nullptr, LNH_ERR_INVALID, buf);
+        }
+    }
+    return LNH_OK;
+}
+
+size_t lnh_row_bytes(uint32_t type, size_t cols) { return nh::gguf_row_bytes(type, cols); }
+
+}  // extern "C"

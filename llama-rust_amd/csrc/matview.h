@@ -1,0 +1,118 @@
+// Device-resident layout of one packed matrix and the per-dtype geometry.
+//
+// A GGUF tensor arrives as an array of self-contained blocks (scale(s) next to
+// the codes they scale; 18/22/24/34/144/210 bytes each, only 2-byte aligned).
+// That is the right layout for a CPU that walks one row with one thread, and
+// the wrong one for a wavefront: 16-byte lane loads straddle block headers and
+// every lane has to pick its codes out of a header/payload mix.  At upload the
+// same bits are therefore re-laid into planes (structure of arrays), per row:
+//
+//   Q8_0 : codes[nb][32]                      | d[nb] f16
+//   Q4_0 : codes[nb][16]                      | d[nb] f16
+//   Q5_0 : codes[nb][16] | qh[nb] u32         | d[nb] f16
+//   Q5_1 : codes[nb][16] | qh[nb] u32         | (d, m)[nb] 2 x f16
+//   Q4_K : codes[nb][128]                     | header[nb][16] = d, dmin, scales[12]
+//   Q6_K : ql[nb][128] | qh[nb][64] | sc[nb][16] int8 | d[nb] f16
+//   F16 / F32 : the row itself, zero-padded to a multiple of 8 elements
+//
+// Nothing is expanded: the planes hold exactly the bytes of the GGUF blocks
+// (F16/F32 rows gain at most 7 elements of zero padding), every code plane row
+// starts 16-byte aligned, and a wavefront's 64 x 16-byte load is one contiguous
+// kilobyte of a single row.
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+namespace nh {
+
+enum : uint32_t {
+    T_F32 = 0,
+    T_F16 = 1,
+    T_Q4_0 = 2,
+    T_Q5_0 = 6,
+    T_Q5_1 = 7,
+    T_Q8_0 = 8,
+    T_Q4_K = 12,
+    T_Q6_K = 14
+};
+
+struct MatView {
+    const uint8_t *p0, *p1, *p2, *p3;  // plane base pointers (device)
+    uint32_t s0, s1, s2, s3;           // plane row strides in bytes
+    uint32_t type, rows, cols, nb;     // nb = blocks per row
+};
+
+inline bool type_supported(uint32_t t) {
+    return t == T_F32 || t == T_F16 || t == T_Q4_0 || t == T_Q5_0 || t == T_Q5_1 || t == T_Q8_0 ||
+           t == T_Q4_K || t == T_Q6_K;
+}
+inline size_t block_elems(uint32_t t) {
+    switch (t) {
+    case T_F32:
+    case T_F16: return 1;
+    case T_Q4_0:
+    case T_Q5_0:
+    case T_Q5_1:
+    case T_Q8_0: return 32;
+    case T_Q4_K:
+    case T_Q6_K: return 256;
+    default: return 0;
+    }
+}
+inline size_t block_bytes(uint32_t t) {
+    switch (t) {
+    case T_F32: return 4;
+    case T_F16: return 2;
+    case T_Q4_0: return 18;
+    case T_Q5_0: return 22;
+    case T_Q5_1: return 24;
+    case T_Q8_0: return 34;
+    case T_Q4_K: return 144;
+    case T_Q6_K: return 210;
+    default: return 0;
+    }
+}
+// Bytes of one GGUF row, 0 when cols is not a whole number of blocks or on overflow.
+inline size_t gguf_row_bytes(uint32_t t, size_t cols) {
+    size_t qk = block_elems(t), bb = block_bytes(t);
+    if (qk == 0 || cols % qk != 0) return 0;
+    size_t nb = cols / qk;
+    if (nb != 0 && bb > SIZE_MAX / nb) return 0;
+    return nb * bb;
+}
+
+struct PlaneSpec {
+    size_t stride[4];  // row strides
+    size_t offset[4];  // plane offsets inside the allocation (256-byte aligned)
+    size_t total;      // allocation size
+};
+
+inline size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Plane geometry for a rows x cols matrix of type t (cols already validated).
+inline PlaneSpec plane_spec(uint32_t t, size_t rows, size_t cols) {
+    PlaneSpec s = {};
+    size_t nb = cols / block_elems(t);
+    switch (t) {
+    case T_F32: s.stride[0] = round_up(cols, 8) * 4; break;  // 8-element groups never leave the row
+    case T_F16: s.stride[0] = round_up(cols, 8) * 2; break;
+    case T_Q8_0: s.stride[0] = nb * 32; s.stride[1] = nb * 2; break;
+    case T_Q4_0: s.stride[0] = nb * 16; s.stride[1] = nb * 2; break;
+    case T_Q5_0: s.stride[0] = nb * 16; s.stride[1] = nb * 4; s.stride[2] = nb * 2; break;
+    case T_Q5_1: s.stride[0] = nb * 16; s.stride[1] = nb * 4; s.stride[2] = nb * 4; break;
+    case T_Q4_K: s.stride[0] = nb * 128; s.stride[1] = nb * 16; break;
+    case T_Q6_K: s.stride[0] = nb * 128; s.stride[1] = nb * 64; s.stride[2] = nb * 16; s.stride[3] = nb * 2; break;
+    default: break;
+    }
+    size_t off = 0;
+    for (int i = 0; i < 4; i++) {
+        s.offset[i] = off;
+        // 64 bytes of slack after every plane: kernels may issue (masked-out) full-width
+        // loads that start inside the last row.
+        off = round_up(off + s.stride[i] * rows + 64, 256);
+    }
+    s.total = off;
+    return s;
+}
+
+}  // namespace nh

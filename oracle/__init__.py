@@ -55,6 +55,8 @@ def load():
                              u8p, C.c_size_t, f32p, C.c_size_t, f32p, C.c_size_t]
     lib.lro_gemm_f64.restype = C.c_int
     lib.lro_gemm_f64.argtypes = [C.c_int, C.c_size_t, C.c_size_t, C.c_size_t, u8p, f32p, f64p]
+    lib.lro_gemm_f64_mag.restype = C.c_int
+    lib.lro_gemm_f64_mag.argtypes = [C.c_int, C.c_size_t, C.c_size_t, C.c_size_t, u8p, f32p, f64p, f64p]
     lib.lro_worker_count.restype = C.c_int
     lib.lro_worker_count.argtypes = [C.c_size_t]
     lib.lro_pack_q8_0_block.argtypes = [C.c_float, u8p, u8p]
@@ -151,6 +153,17 @@ def gemm_f64(ty, n_cols, n_tokens, w, x, n_rows):
     if rc != 0:
         raise ValueError(f"lro_gemm_f64 failed: {rc}")
     return y.reshape(n_tokens, n_rows)
+
+
+def gemm_f64_mag(ty, n_cols, n_tokens, w, x, n_rows):
+    """(exact-ish f64 product, sum |w||x| per output), both token-major [n_tokens, n_rows]."""
+    w, x = _u8(w), _f32(x)
+    y = np.empty(n_tokens * n_rows, dtype=np.float64)
+    mag = np.empty(n_tokens * n_rows, dtype=np.float64)
+    rc = load().lro_gemm_f64_mag(ty, n_cols, n_tokens, n_rows, _p(w), _p(x), _p(y), _p(mag))
+    if rc != 0:
+        raise ValueError(f"lro_gemm_f64_mag failed: {rc}")
+    return y.reshape(n_tokens, n_rows), mag.reshape(n_tokens, n_rows)
 
 
 def validate(actual, expected):

@@ -381,6 +381,34 @@ int lro_gemm_f64(int type, size_t n_cols, size_t n_tokens, size_t n_rows, const 
     return 0;
 }
 
+/* f64 product and the magnitude sum |w||x| of every output in one pass. */
+int lro_gemm_f64_mag(int type, size_t n_cols, size_t n_tokens, size_t n_rows, const uint8_t *w,
+                     const float *x, double *y, double *mag) {
+    size_t rb = lro_row_bytes(type, n_cols);
+    if (rb == 0 && n_cols != 0) return -1;
+    float *wr = (float *)malloc((n_cols ? n_cols : 1) * sizeof(float));
+    if (!wr) return -2;
+    for (size_t r = 0; r < n_rows; r++) {
+        if (lro_dequant_row(type, n_cols, w + r * rb, wr) != 0) {
+            free(wr);
+            return -1;
+        }
+        for (size_t t = 0; t < n_tokens; t++) {
+            const float *xt = x + t * n_cols;
+            double s = 0.0, a = 0.0;
+            for (size_t c = 0; c < n_cols; c++) {
+                double p = (double)wr[c] * (double)xt[c];
+                s += p;
+                a += fabs(p);
+            }
+            y[t * n_rows + r] = s;
+            mag[t * n_rows + r] = a;
+        }
+    }
+    free(wr);
+    return 0;
+}
+
 /* ---------------------------------------------------------------- threaded GEMM */
 
 /* langtax/src/pool.rs:43, 70-79 */

@@ -90,6 +90,10 @@ int lro_gemm(int type, int kind, int threads, size_t n_cols, size_t n_tokens,
 /* Same product as exact-as-possible f64 sums over the dequantized weights. */
 int lro_gemm_f64(int type, size_t n_cols, size_t n_tokens, size_t n_rows,
                  const uint8_t *w, const float *x, double *y);
+/* The f64 product together with sum_c |W[r,c] x[t,c]| per output (the scale of
+ * the reference's error bound, langtax/src/simd/tests.rs:93-105). */
+int lro_gemm_f64_mag(int type, size_t n_cols, size_t n_tokens, size_t n_rows, const uint8_t *w,
+                     const float *x, double *y, double *mag);
 /* Worker count the reference would use for n_rows rows (pool.rs:70-79). */
 int lro_worker_count(size_t n_rows);
 
