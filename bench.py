@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Benchmark of the decode GEMV hot path on one MI355X.
+
+Workload (BASELINE config "Llama-3-8B decode layer shapes as batch-1 GEMV"): one
+step is one generated token's weight products, batch 1 - for each of 32 layers
+the seven Q4_K GEMVs q, k, v, o (4096->4096/1024), gate, up (4096->14336), down
+(14336->4096), then the Q6_K output head 4096->128256 - 225 products streaming
+4.36 GB of distinct packed weights, so no product is served from the 256 MB
+Infinity Cache.  Activations and outputs stay resident in HBM; weights are
+synthetic (uniform codes, |N(0, 0.02)| f16 block scales), x ~ N(0, 1).
+
+`value` is algorithmic bytes per step / wall time per step.  `roofline` is for the
+dominant kernel (the Q4_K GEMV, 224 launches per step): algorithmic bytes per
+launch / mean launch duration from HIP events recorded on the launch stream
+around the Q4_K part of every timed step.  `cpu_baseline` times the AVX2 port of
+the reference's `simd` CPU kernels on a bounded sample of the same workload.
+
+One JSON line on stdout; progress on stderr.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "Q4_K/Q8_0 GEMV HBM GB/s (% of peak); 8B-shape decode tok/s, batch 1"
+HBM_PEAK_GBS = 8000.0
+Q4_K, Q6_K = 12, 14
+N_LAYERS, D, D_KV, FF, VOCAB = 32, 4096, 1024, 14336, 128256
+LAYER = [("q", D, D), ("k", D_KV, D), ("v", D_KV, D), ("o", D, D), ("gate", FF, D), ("up", FF, D), ("down", D, FF)]
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def row_bytes(ty, cols):
+    return cols // 256 * (144 if ty == Q4_K else 210)
+
+
+def algorithmic_bytes(ty, rows, cols, tokens=1):
+    """Each weight byte once, x once, y once."""
+    return rows * row_bytes(ty, cols) + 4 * tokens * cols + 4 * tokens * rows
+
+
+def synth_matrix(ty, rows, cols, rng):
+    """Packed GGUF bytes: uniform random codes / 6-bit scales, |N(0, 0.02)| f16 super-block scales."""
+    nb = cols // 256
+    bb = 144 if ty == Q4_K else 210
+    blk = rng.integers(0, 256, size=(rows, nb, bb), dtype=np.uint8)
+    if ty == Q4_K:
+        blk[:, :, 0:4] = np.abs(rng.normal(0, 0.02, (rows, nb, 2))).astype(np.float16).view(np.uint8).reshape(rows, nb, 4)
+    else:
+        blk[:, :, 208:210] = np.abs(rng.normal(0, 0.02, (rows, nb, 1))).astype(np.float16).view(np.uint8).reshape(rows, nb, 2)
+    return blk.reshape(-1)
+
+
+def cpu_baseline(sample, x_by_cols, seconds):
+    """The reference's `simd` CPU path (AVX2 port, <=10 threads, fork/join per product)
+    on `sample` = [(type, rows, cols, packed bytes)], repeated for about `seconds`."""
+    import oracle as O
+    threads = O.load().lro_worker_count(1 << 20)
+    nbytes = sum(algorithmic_bytes(ty, r, c) for ty, r, c, _ in sample)
+
+    def sweep():
+        for ty, r, c, w in sample:
+            O.gemm(ty, c, 1, w, x_by_cols[c], r, simd=True, threads=0)
+
+    sweep()  # warm-up
+    t0 = time.perf_counter()
+    n = 0
+    while True:
+        sweep()
+        n += 1
+        dt = time.perf_counter() - t0
+        if dt >= seconds or n >= 2000:
+            break
+    return {"value": nbytes * n / dt / 1e9, "unit": "GB/s", "cores": int(threads), "kind": "port",
+            "sample": f"layer 0 (7 Q4_K GEMVs) + first {sample[-1][1]} rows of the Q6_K head, "
+                      f"{nbytes / 1e6:.1f} MB per sweep, {n} sweeps in {dt:.1f} s, AVX2 port of the reference simd kernels",
+            "tok_per_s_equiv": n / dt * nbytes / TOKEN_BYTES}
+
+
+TOKEN_BYTES = N_LAYERS * sum(algorithmic_bytes(Q4_K, r, c) for _, r, c in LAYER) + algorithmic_bytes(Q6_K, VOCAB, D)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=N_LAYERS, help="fewer layers only for quick experiments")
+    ap.add_argument("--no-graph", action="store_true", help="enqueue every product eagerly instead of replaying HIP graphs")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="0 skips the CPU baseline")
+    ap.add_argument("--seed", type=int, default=20240531)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); "
+            "the path shards by weight rows, which is described in DESIGN.md but not built")
+        return 2
+
+    pkg = importlib.import_module("llama-rust_amd")
+    hip = importlib.import_module("llama-rust_amd.hiprt")
+    gpu = pkg.HipGemv(0)
+    rng = np.random.default_rng(args.seed)
+
+    t_setup = time.perf_counter()
+    x_host = {D: rng.normal(0, 1, D).astype(np.float32), FF: rng.normal(0, 1, FF).astype(np.float32)}
+    x_dev = {c: hip.DeviceBuffer.from_numpy(v) for c, v in x_host.items()}
+    mats, xs, ys, keep = [], [], [], []
+    sample = []
+    y_bufs = {}
+    for layer in range(args.layers):
+        for name, rows, cols in LAYER:
+            w = synth_matrix(Q4_K, rows, cols, rng)
+            mats.append(gpu.upload_packed(Q4_K, rows, cols, w))
+            xs.append(x_dev[cols].ptr)
+            slot = 0 if layer == 0 else 1 + layer % 2   # layer 0 keeps its outputs for the sanity check
+            if (slot, name) not in y_bufs:
+                y_bufs[(slot, name)] = hip.DeviceBuffer(rows * 4)
+            ys.append(y_bufs[(slot, name)].ptr)
+            if layer == 0:
+                sample.append((Q4_K, rows, cols, w))
+        if layer % 8 == 7:
+            log(f"[bench] uploaded {layer + 1}/{args.layers} layers ({time.perf_counter() - t_setup:.1f} s)")
+    head_w = synth_matrix(Q6_K, VOCAB, D, rng)
+    head = gpu.upload_packed(Q6_K, VOCAB, D, head_w)
+    head_rows = VOCAB // 16
+    sample.append((Q6_K, head_rows, D, head_w[:head_rows * row_bytes(Q6_K, D)].copy()))
+    head_y = hip.DeviceBuffer(VOCAB * 4)
+    del head_w
+    n_q4k = len(mats)
+    log(f"[bench] {n_q4k} Q4_K matrices + Q6_K head resident, setup {time.perf_counter() - t_setup:.1f} s")
+
+    stream = hip.Stream()
+    layers_batch = gpu.make_batch(mats, [1] * n_q4k, xs, ys)
+    head_batch = gpu.make_batch([head], [1], [x_dev[D].ptr], [head_y.ptr])
+    enqueue_layers = lambda s=stream: gpu.gemm_batch_device(layers_batch, s.ptr)
+    enqueue_head = lambda s=stream: gpu.gemm_batch_device(head_batch, s.ptr)
+    enqueue_layers(); enqueue_head(); stream.synchronize()       # first launches configure the kernels
+    if not args.no_graph:
+        g_layers = hip.Graph(stream, enqueue_layers)
+        g_head = hip.Graph(stream, enqueue_head)
+        run_layers, run_head = g_layers.launch, g_head.launch
+    else:
+        run_layers, run_head = enqueue_layers, enqueue_head
+
+    # sanity: a sample of layer-0 outputs against the CPU oracle before timing anything
+    import oracle as O
+    run_layers(); run_head(); stream.synchronize()
+    ty, rows, cols, w = sample[0]
+    got = y_bufs[(0, "q")].to_numpy(np.float32)[:64]
+    want = O.gemm_f64(ty, cols, 1, w[:64 * row_bytes(ty, cols)], x_host[cols], 64)[0]
+    if not np.allclose(got, want, rtol=1e-4, atol=1e-4 * float(np.sqrt(np.mean(want ** 2)))):
+        log("[bench] FATAL: GPU output disagrees with the CPU oracle")
+        return 1
+
+    for _ in range(args.warmup):
+        run_layers(); run_head()
+    stream.synchronize()
+
+    ev = [(hip.Event(), hip.Event(), hip.Event()) for _ in range(args.steps)]
+    hip.device_synchronize()
+    t0 = time.perf_counter()
+    for a, b, c in ev:
+        a.record(stream)
+        run_layers()
+        b.record(stream)
+        run_head()
+        c.record(stream)
+    stream.synchronize()
+    hip.device_synchronize()
+    wall = time.perf_counter() - t0
+
+    q4k_ms = sum(a.elapsed_ms(b) for a, b, _ in ev)
+    head_ms = sum(b.elapsed_ms(c) for _, b, c in ev)
+    q4k_bytes = (args.layers * sum(algorithmic_bytes(Q4_K, r, c) for _, r, c in LAYER))
+    head_bytes = algorithmic_bytes(Q6_K, VOCAB, D)
+    step_bytes = q4k_bytes + head_bytes
+    ms_per_step = wall * 1e3 / args.steps
+    value = step_bytes / (wall / args.steps) / 1e9
+    q4k_launch_us = q4k_ms * 1e3 / (args.steps * n_q4k)
+    q4k_gbs = q4k_bytes / (q4k_ms / args.steps * 1e-3) / 1e9
+    head_gbs = head_bytes / (head_ms / args.steps * 1e-3) / 1e9
+
+    out = {
+        "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"Llama-3-8B decode GEMV, batch 1: {args.layers} layers x 7 Q4_K products + Q6_K head 4096->128256",
+                   "weights_gb": round(step_bytes / 1e9, 3), "launches_per_step": n_q4k + 1,
+                   "launch_mode": "eager" if args.no_graph else "hip_graph"},
+        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+        "tok_per_s": round(args.steps / wall, 1),
+        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<Q4_K>", "achieved": round(q4k_gbs, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(q4k_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "bytes_per_launch": round(q4k_bytes / n_q4k), "launch_us": round(q4k_launch_us, 3),
+                     "launches_timed": args.steps * n_q4k},
+        "other_kernels": {"gemv_kernel<Q6_K> head": {"achieved": round(head_gbs, 1), "unit": "GB/s",
+                                                     "frac": round(head_gbs / HBM_PEAK_GBS, 4),
+                                                     "launch_us": round(head_ms * 1e3 / args.steps, 2)}},
+    }
+    if args.cpu_seconds > 0:
+        log("[bench] timing the CPU baseline ...")
+        out["cpu_baseline"] = cpu_baseline(sample, x_host, args.cpu_seconds)
+        out["cpu_baseline"]["value"] = round(out["cpu_baseline"]["value"], 2)
+        out["cpu_baseline"]["tok_per_s_equiv"] = round(out["cpu_baseline"]["tok_per_s_equiv"], 3)
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

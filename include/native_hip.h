@@ -118,6 +118,12 @@ int lnh_gemm_device(lnh_exec *exec, const lnh_matrix *matrix, size_t tokens, con
                     float *device_y, void *stream);
 int lnh_gemm_grouped_device(lnh_exec *exec, size_t n_groups, const lnh_matrix *const *mats,
                             const size_t *tokens, const float *device_x, float *device_y, void *stream);
+/* n independent products enqueued back to back in one call: product i multiplies
+ * tokens[i] rows at device_x[i] by mats[i] into device_y[i].  This is how a decode
+ * step's products (langtax/src/decode.rs:2755-2996: q, k, v, o, gate, up, down per
+ * layer) are issued without a host round trip each. */
+int lnh_gemm_batch_device(lnh_exec *exec, size_t n, const lnh_matrix *const *mats, const size_t *tokens,
+                          const float *const *device_x, float *const *device_y, void *stream);
 /* Block the host until everything enqueued on the executor's own stream is done. */
 int lnh_synchronize(lnh_exec *exec);
 

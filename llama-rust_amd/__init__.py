@@ -88,6 +88,7 @@ def load_library():
         "lnh_gemm_grouped": (C.c_int, [vp, sz, pvp, psz, vp, sz, vp, sz]),
         "lnh_gemm_device": (C.c_int, [vp, vp, sz, vp, vp, vp]),
         "lnh_gemm_grouped_device": (C.c_int, [vp, sz, pvp, psz, vp, vp, vp]),
+        "lnh_gemm_batch_device": (C.c_int, [vp, sz, pvp, psz, pvp, pvp, vp]),
         "lnh_synchronize": (C.c_int, [vp]),
         "lnh_shape_checked": (C.c_int, [sz, sz, sz, sz, C.POINTER(u32), C.POINTER(u32)]),
         "lnh_validate": (C.c_int, [vp, sz, vp, sz]),
@@ -267,6 +268,16 @@ class HipGemv:
         toks = (C.c_size_t * n)(*tokens)
         self._check(self._lib.lnh_gemm_grouped_device(self._h, n, mats, toks, C.c_void_p(x_ptr), C.c_void_p(y_ptr),
                                                       C.c_void_p(stream)))
+
+    def make_batch(self, matrices, tokens, x_ptrs, y_ptrs):
+        """Pre-marshalled argument arrays for gemm_batch_device (reused across calls)."""
+        n = len(matrices)
+        return (n, (C.c_void_p * n)(*[m._h for m in matrices]), (C.c_size_t * n)(*tokens),
+                (C.c_void_p * n)(*x_ptrs), (C.c_void_p * n)(*y_ptrs))
+
+    def gemm_batch_device(self, batch, stream=0):
+        n, mats, toks, xs, ys = batch
+        self._check(self._lib.lnh_gemm_batch_device(self._h, n, mats, toks, xs, ys, C.c_void_p(stream)))
 
     def synchronize(self):
         self._check(self._lib.lnh_synchronize(self._h))

@@ -413,6 +413,24 @@ int lnh_gemm_grouped_device(lnh_exec *e, size_t n_groups, const lnh_matrix *cons
     return LNH_OK;
 }
 
+int lnh_gemm_batch_device(lnh_exec *e, size_t n, const lnh_matrix *const *mats, const size_t *tokens,
+                          const float *const *dx, float *const *dy, void *stream) {
+    if (!e) return LNH_ERR_INVALID;
+    if (n != 0 && (!mats || !tokens || !dx || !dy)) return fail(e, LNH_ERR_INVALID, "batch arrays are null");
+    for (size_t i = 0; i < n; i++) {  // validate everything before the first launch
+        size_t inputs, outputs;
+        int rc = check_gemm(e, mats[i], tokens[i], false, 0, 0, &inputs, &outputs);
+        if (rc != LNH_OK) return rc;
+        if (!dx[i] || !dy[i]) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    }
+    hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
+    for (size_t i = 0; i < n; i++) {
+        hipError_t h = nh::launch_gemm(s, mats[i]->view, (uint32_t)tokens[i], dx[i], dy[i]);
+        if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
+    }
+    return LNH_OK;
+}
+
 int lnh_synchronize(lnh_exec *e) {
     if (!e) return LNH_ERR_INVALID;
     hipError_t h = hipStreamSynchronize(e->stream);

@@ -36,6 +36,12 @@ def rt():
         lib.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
         lib.hipEventDestroy.argtypes = [C.c_void_p]
         lib.hipSetDevice.argtypes = [C.c_int]
+        lib.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+        lib.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        lib.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+        lib.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+        lib.hipGraphExecDestroy.argtypes = [C.c_void_p]
+        lib.hipGraphDestroy.argtypes = [C.c_void_p]
         _rt = lib
     return _rt
 
@@ -117,6 +123,33 @@ class Event:
         if self.ptr:
             rt().hipEventDestroy(self.ptr)
             self.ptr = None
+
+
+class Graph:
+    """A stream capture of whatever `enqueue(stream)` launches, replayable with launch()."""
+
+    def __init__(self, stream, enqueue):
+        check(rt().hipStreamBeginCapture(stream.ptr, 0), "hipStreamBeginCapture")  # global mode
+        try:
+            enqueue(stream)
+        finally:
+            g = C.c_void_p()
+            code = rt().hipStreamEndCapture(stream.ptr, C.byref(g))
+        check(code, "hipStreamEndCapture")
+        self.graph = g.value
+        ex = C.c_void_p()
+        check(rt().hipGraphInstantiate(C.byref(ex), self.graph, None, None, 0), "hipGraphInstantiate")
+        self.exec = ex.value
+        self.stream = stream
+
+    def launch(self):
+        check(rt().hipGraphLaunch(self.exec, self.stream.ptr), "hipGraphLaunch")
+
+    def destroy(self):
+        if self.exec:
+            rt().hipGraphExecDestroy(self.exec)
+            rt().hipGraphDestroy(self.graph)
+            self.exec = self.graph = None
 
 
 def device_synchronize():
