@@ -10,7 +10,8 @@ Infinity Cache.  Activations and outputs stay resident in HBM; weights are
 synthetic (uniform codes, |N(0, 0.02)| f16 block scales), x ~ N(0, 1).
 
 `value` is algorithmic bytes per step / wall time per step.  `roofline` is for the
-dominant kernel (the Q4_K GEMV, 224 launches per step): algorithmic bytes per
+dominant kernel (the Q4_K GEMV: 224 products in 128 launches per step, products that
+share an input vector - q/k/v, gate/up - being one launch): algorithmic bytes per
 launch / mean launch duration from HIP events recorded on the launch stream
 around the Q4_K part of every timed step.  `cpu_baseline` times the AVX2 port of
 the reference's `simd` CPU kernels on a bounded sample of the same workload.
@@ -33,7 +34,13 @@ METRIC = "Q4_K/Q8_0 GEMV HBM GB/s (% of peak); 8B-shape decode tok/s, batch 1"
 HBM_PEAK_GBS = 8000.0
 Q4_K, Q6_K = 12, 14
 N_LAYERS, D, D_KV, FF, VOCAB = 32, 4096, 1024, 14336, 128256
-LAYER = [("q", D, D), ("k", D_KV, D), ("v", D_KV, D), ("o", D, D), ("gate", FF, D), ("up", FF, D), ("down", D, FF)]
+# (name, rows, cols, which activation buffer it reads).  Products that read the same buffer are
+# independent of each other (q/k/v of the normed hidden state, gate/up of the normed residual);
+# o and down read what the host computes from the earlier products, so they are launches of
+# their own.  lnh_gemm_batch_device issues each run of same-input products as one launch.
+LAYER = [("q", D, D, "h1"), ("k", D_KV, D, "h1"), ("v", D_KV, D, "h1"), ("o", D, D, "attn"),
+         ("gate", FF, D, "h2"), ("up", FF, D, "h2"), ("down", D, FF, "act")]
+LAUNCHES_PER_LAYER = 4
 
 
 def log(*a):
@@ -66,11 +73,11 @@ def cpu_baseline(sample, x_by_cols, seconds):
     on `sample` = [(type, rows, cols, packed bytes)], repeated for about `seconds`."""
     import oracle as O
     threads = O.load().lro_worker_count(1 << 20)
-    nbytes = sum(algorithmic_bytes(ty, r, c) for ty, r, c, _ in sample)
+    nbytes = sum(algorithmic_bytes(ty, r, c) for ty, r, c, _, _ in sample)
 
     def sweep():
-        for ty, r, c, w in sample:
-            O.gemm(ty, c, 1, w, x_by_cols[c], r, simd=True, threads=0)
+        for ty, r, c, w, src in sample:
+            O.gemm(ty, c, 1, w, x_by_cols[src], r, simd=True, threads=0)
 
     sweep()  # warm-up
     t0 = time.perf_counter()
@@ -87,7 +94,7 @@ def cpu_baseline(sample, x_by_cols, seconds):
             "tok_per_s_equiv": n / dt * nbytes / TOKEN_BYTES}
 
 
-TOKEN_BYTES = N_LAYERS * sum(algorithmic_bytes(Q4_K, r, c) for _, r, c in LAYER) + algorithmic_bytes(Q6_K, VOCAB, D)
+TOKEN_BYTES = N_LAYERS * sum(algorithmic_bytes(Q4_K, r, c) for _, r, c, _ in LAYER) + algorithmic_bytes(Q6_K, VOCAB, D)
 
 
 def main():
@@ -111,28 +118,29 @@ def main():
     rng = np.random.default_rng(args.seed)
 
     t_setup = time.perf_counter()
-    x_host = {D: rng.normal(0, 1, D).astype(np.float32), FF: rng.normal(0, 1, FF).astype(np.float32)}
-    x_dev = {c: hip.DeviceBuffer.from_numpy(v) for c, v in x_host.items()}
+    x_host = {"h1": rng.normal(0, 1, D).astype(np.float32), "attn": rng.normal(0, 1, D).astype(np.float32),
+              "h2": rng.normal(0, 1, D).astype(np.float32), "act": rng.normal(0, 1, FF).astype(np.float32)}
+    x_dev = {k: hip.DeviceBuffer.from_numpy(v) for k, v in x_host.items()}
     mats, xs, ys, keep = [], [], [], []
     sample = []
     y_bufs = {}
     for layer in range(args.layers):
-        for name, rows, cols in LAYER:
+        for name, rows, cols, src in LAYER:
             w = synth_matrix(Q4_K, rows, cols, rng)
             mats.append(gpu.upload_packed(Q4_K, rows, cols, w))
-            xs.append(x_dev[cols].ptr)
+            xs.append(x_dev[src].ptr)
             slot = 0 if layer == 0 else 1 + layer % 2   # layer 0 keeps its outputs for the sanity check
             if (slot, name) not in y_bufs:
                 y_bufs[(slot, name)] = hip.DeviceBuffer(rows * 4)
             ys.append(y_bufs[(slot, name)].ptr)
             if layer == 0:
-                sample.append((Q4_K, rows, cols, w))
+                sample.append((Q4_K, rows, cols, w, src))
         if layer % 8 == 7:
             log(f"[bench] uploaded {layer + 1}/{args.layers} layers ({time.perf_counter() - t_setup:.1f} s)")
     head_w = synth_matrix(Q6_K, VOCAB, D, rng)
     head = gpu.upload_packed(Q6_K, VOCAB, D, head_w)
     head_rows = VOCAB // 16
-    sample.append((Q6_K, head_rows, D, head_w[:head_rows * row_bytes(Q6_K, D)].copy()))
+    sample.append((Q6_K, head_rows, D, head_w[:head_rows * row_bytes(Q6_K, D)].copy(), "h1"))
     head_y = hip.DeviceBuffer(VOCAB * 4)
     del head_w
     n_q4k = len(mats)
@@ -140,7 +148,7 @@ def main():
 
     stream = hip.Stream()
     layers_batch = gpu.make_batch(mats, [1] * n_q4k, xs, ys)
-    head_batch = gpu.make_batch([head], [1], [x_dev[D].ptr], [head_y.ptr])
+    head_batch = gpu.make_batch([head], [1], [x_dev["h1"].ptr], [head_y.ptr])
     enqueue_layers = lambda s=stream: gpu.gemm_batch_device(layers_batch, s.ptr)
     enqueue_head = lambda s=stream: gpu.gemm_batch_device(head_batch, s.ptr)
     enqueue_layers(); enqueue_head(); stream.synchronize()       # first launches configure the kernels
@@ -154,12 +162,12 @@ def main():
     # sanity: a sample of layer-0 outputs against the CPU oracle before timing anything
     import oracle as O
     run_layers(); run_head(); stream.synchronize()
-    ty, rows, cols, w = sample[0]
-    got = y_bufs[(0, "q")].to_numpy(np.float32)[:64]
-    want = O.gemm_f64(ty, cols, 1, w[:64 * row_bytes(ty, cols)], x_host[cols], 64)[0]
-    if not np.allclose(got, want, rtol=1e-4, atol=1e-4 * float(np.sqrt(np.mean(want ** 2)))):
-        log("[bench] FATAL: GPU output disagrees with the CPU oracle")
-        return 1
+    for (ty, rows, cols, w, src), (name, _, _, _) in zip(sample, LAYER):
+        got = y_bufs[(0, name)].to_numpy(np.float32)[:64]
+        want = O.gemm_f64(ty, cols, 1, w[:64 * row_bytes(ty, cols)], x_host[src], 64)[0]
+        if not np.allclose(got, want, rtol=1e-4, atol=1e-4 * float(np.sqrt(np.mean(want ** 2)))):
+            log(f"[bench] FATAL: GPU output of layer-0 {name} disagrees with the CPU oracle")
+            return 1
 
     for _ in range(args.warmup):
         run_layers(); run_head()
@@ -180,12 +188,13 @@ def main():
 
     q4k_ms = sum(a.elapsed_ms(b) for a, b, _ in ev)
     head_ms = sum(b.elapsed_ms(c) for _, b, c in ev)
-    q4k_bytes = (args.layers * sum(algorithmic_bytes(Q4_K, r, c) for _, r, c in LAYER))
+    q4k_bytes = (args.layers * sum(algorithmic_bytes(Q4_K, r, c) for _, r, c, _ in LAYER))
+    n_launch = args.layers * LAUNCHES_PER_LAYER
     head_bytes = algorithmic_bytes(Q6_K, VOCAB, D)
     step_bytes = q4k_bytes + head_bytes
     ms_per_step = wall * 1e3 / args.steps
     value = step_bytes / (wall / args.steps) / 1e9
-    q4k_launch_us = q4k_ms * 1e3 / (args.steps * n_q4k)
+    q4k_launch_us = q4k_ms * 1e3 / (args.steps * n_launch)
     q4k_gbs = q4k_bytes / (q4k_ms / args.steps * 1e-3) / 1e9
     head_gbs = head_bytes / (head_ms / args.steps * 1e-3) / 1e9
 
@@ -194,14 +203,15 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"Llama-3-8B decode GEMV, batch 1: {args.layers} layers x 7 Q4_K products + Q6_K head 4096->128256",
-                   "weights_gb": round(step_bytes / 1e9, 3), "launches_per_step": n_q4k + 1,
+                   "weights_gb": round(step_bytes / 1e9, 3), "products_per_step": n_q4k + 1, "launches_per_step": n_launch + 1,
+                   "launch_grouping": "per layer [q,k,v] [o] [gate,up] [down]: products sharing an input are one launch",
                    "launch_mode": "eager" if args.no_graph else "hip_graph"},
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "tok_per_s": round(args.steps / wall, 1),
-        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<Q4_K>", "achieved": round(q4k_gbs, 1), "peak": HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": "gemv_q4k_kernel", "achieved": round(q4k_gbs, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(q4k_gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "bytes_per_launch": round(q4k_bytes / n_q4k), "launch_us": round(q4k_launch_us, 3),
-                     "launches_timed": args.steps * n_q4k},
+                     "bytes_per_launch": round(q4k_bytes / n_launch), "launch_us": round(q4k_launch_us, 3),
+                     "launches_timed": args.steps * n_launch},
         "other_kernels": {"gemv_kernel<Q6_K> head": {"achieved": round(head_gbs, 1), "unit": "GB/s",
                                                      "frac": round(head_gbs / HBM_PEAK_GBS, 4),
                                                      "launch_us": round(head_ms * 1e3 / args.steps, 2)}},

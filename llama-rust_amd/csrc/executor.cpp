@@ -242,6 +242,13 @@ int lnh_create(int device_ordinal, lnh_exec **out) {
     e->ctx->id = g_next_ctx.fetch_add(1);
     h = hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking);
     if (h != hipSuccess) return hip_fail(nullptr, h, "hipStreamCreate");
+    float unit = 0.f;
+    h = nh::probe_fp8_nibble_unit(e->stream, &unit);
+    if (h != hipSuccess) {
+        (void)hipStreamDestroy(e->stream);
+        return hip_fail(nullptr, h, "fp8 unpack probe");
+    }
+    nh::set_fp8_nibble_unit(unit);
     *out = e.release();
     return LNH_OK;
 }
@@ -424,9 +431,29 @@ int lnh_gemm_batch_device(lnh_exec *e, size_t n, const lnh_matrix *const *mats, 
         if (!dx[i] || !dy[i]) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
     }
     hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
-    for (size_t i = 0; i < n; i++) {
-        hipError_t h = nh::launch_gemm(s, mats[i]->view, (uint32_t)tokens[i], dx[i], dy[i]);
+    for (size_t i = 0; i < n;) {
+        // Single-token products that read the same x (q/k/v, gate/up) go out as one launch.
+        size_t run = 1;
+        while (tokens[i] == 1 && i + run < n && run < 8 && tokens[i + run] == 1 && dx[i + run] == dx[i] &&
+               mats[i + run]->view.type == mats[i]->view.type && mats[i + run]->view.cols == mats[i]->view.cols)
+            run++;
+        hipError_t h = hipErrorInvalidValue;
+        if (run > 1) {
+            nh::MatView views[8];
+            float *ys[8];
+            for (size_t k = 0; k < run; k++) {
+                views[k] = mats[i + k]->view;
+                ys[k] = dy[i + k];
+            }
+            h = nh::launch_gemv_multi(s, views, ys, (uint32_t)run, dx[i]);
+            if (h == hipErrorInvalidValue) (void)hipGetLastError();
+        }
+        if (h == hipErrorInvalidValue) {
+            run = 1;
+            h = nh::launch_gemm(s, mats[i]->view, (uint32_t)tokens[i], dx[i], dy[i]);
+        }
         if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
+        i += run;
     }
     return LNH_OK;
 }

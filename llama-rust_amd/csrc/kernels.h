@@ -9,10 +9,21 @@ namespace nh {
 // CU count and the largest dynamic LDS a workgroup may ask for on this device.
 void set_device_limits(int cu_count, size_t lds_per_block);
 
+// Value the fp8 (E4M3) unpack gives for byte 0x01 on this device when bytes 0..15 decode
+// linearly (n * unit), else 0: nibble kernels then take the byte-convert path.
+void set_fp8_nibble_unit(float unit);
+// Runs a 16-thread probe kernel and reports that unit (0 when the decode is not linear).
+hipError_t probe_fp8_nibble_unit(hipStream_t stream, float *unit_out);
+
 // Scatter the GGUF bytes at src_device (device memory) into the planes of m.
 hipError_t launch_repack(hipStream_t stream, const MatView &m, const void *src_device);
 
 // y[t, r] = sum_c W[r, c] x[t, c]; x and y are device pointers, token-major.
 hipError_t launch_gemm(hipStream_t stream, const MatView &m, uint32_t tokens, const float *x, float *y);
+
+// One launch for up to 8 single-token products that read the same x and share dtype
+// and column count (q/k/v, gate/up).  hipErrorInvalidValue = not fusable this way;
+// the caller then launches them one by one.
+hipError_t launch_gemv_multi(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x);
 
 }  // namespace nh

@@ -10,6 +10,9 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <cmath>
+#include <cstdlib>
+
 #include "kernels.h"
 
 namespace nh {
@@ -118,8 +121,11 @@ __global__ void repack_blocks(MutView v, const uint8_t *__restrict__ src, size_t
         const uint8_t *s = src + r * src_row_bytes + b * 144;
         uint8_t *h = v.p1 + r * v.s1 + b * 16;
         for (int i = 0; i < 16; i++) h[i] = s[i];
-        uint8_t *q = v.p0 + r * v.s0 + b * 128;
-        for (int i = 0; i < 128; i++) q[i] = s[16 + i];
+        // 16-byte piece cc of block b goes to slot cc * nb + b of the row (matview.h)
+        for (int cc = 0; cc < 8; cc++) {
+            uint8_t *q = v.p0 + r * v.s0 + ((size_t)cc * v.nb + b) * 16;
+            for (int i = 0; i < 16; i++) q[i] = s[16 + cc * 16 + i];
+        }
         break;
     }
     case T_Q6_K: {
@@ -278,7 +284,7 @@ template <uint32_t T> __device__ __forceinline__ void load_raw(const MatView &m,
         r.qh = *reinterpret_cast<const uint32_t *>(m.p1 + ro * m.s1 + (size_t)c * 4);
         r.dm = *reinterpret_cast<const uint32_t *>(m.p2 + ro * m.s2 + (size_t)c * 4);
     } else if constexpr (T == T_Q4_K) {
-        r.q = *reinterpret_cast<const uint4 *>(m.p0 + ro * m.s0 + (size_t)c * 16);
+        r.q = *reinterpret_cast<const uint4 *>(m.p0 + ro * m.s0 + ((size_t)(c & 7) * m.nb + (c >> 3)) * 16);
         r.hdr = *reinterpret_cast<const uint4 *>(m.p1 + ro * m.s1 + (size_t)(c >> 3) * 16);
     } else if constexpr (T == T_Q6_K) {
         uint32_t blk = c >> 3, cc = c & 7, n = cc >> 2, k = cc & 1;
@@ -399,68 +405,397 @@ __device__ __forceinline__ float chunk_dot(const Raw<T> &r, const XChunk<Geo<T>:
 
 // ------------------------------------------------------------------ GEMV (one token)
 //
-// One workgroup of NW wavefronts stages x in LDS once, then walks row tiles.
-// Inside a tile, KW wavefronts split the columns of the same R rows (step s of
-// the row belongs to wavefront s mod KW), RW = NW / KW such groups sit side by
-// side on different rows.  Partial sums of the KW wavefronts meet in LDS and are
-// added in a fixed order, so a result never depends on scheduling.
+// Free-running wavefronts.  A workgroup (8 wavefronts) stages x and the
+// per-chunk sums of x in LDS once; after that single barrier every wavefront
+// streams on its own: it owns whole row groups (R consecutive rows, all of
+// their columns), walks them in steps of 64 chunks, and always has the next
+// step's weight bytes in flight while it does the arithmetic of the current one
+// (two register buffers, used alternately).  One DPP reduction per row group,
+// no barrier and no LDS traffic between wavefronts, so the sum of a row is
+// formed in a fixed order that does not depend on scheduling.  One launch can
+// serve several matrices that share the same x (q/k/v, gate/up): row groups of
+// all jobs are numbered consecutively and dealt round-robin to the wavefronts.
 
-template <uint32_t T, int R, int NW>
-__global__ __launch_bounds__(NW * 64) void gemv_kernel(MatView m, const float *__restrict__ x, float *__restrict__ y,
-                                                        uint32_t n_chunks, uint32_t kw_count, uint32_t rw_count,
-                                                        uint32_t x_pad) {
+constexpr int GEMV_WAVES = 8;
+constexpr int GEMV_MAX_JOBS = 8;
+
+struct GemvJob {
+    MatView m;
+    float *y;
+    uint32_t rg_begin;  // first row group of this job in the launch-wide numbering
+    uint32_t pad;
+};
+struct GemvBatch {
+    GemvJob job[GEMV_MAX_JOBS];
+    const float *x;
+    uint32_t n_jobs, total_rgs, n_chunks, x_pad;
+};
+
+template <uint32_t T> __device__ __forceinline__ void load_x_lds(const float *xs, const float *sums, uint32_t c,
+                                                                  XChunk<Geo<T>::E> &o) {
+    constexpr int E = Geo<T>::E;
+    if constexpr (T == T_Q4_K || T == T_Q6_K) {
+        const float4 *lo = reinterpret_cast<const float4 *>(xs + chunk_col<T>(c, 0));
+        const float4 *hi = reinterpret_cast<const float4 *>(xs + chunk_col<T>(c, 16));
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float4 a = lo[i], b = hi[i];
+            o.x[4 * i] = a.x; o.x[4 * i + 1] = a.y; o.x[4 * i + 2] = a.z; o.x[4 * i + 3] = a.w;
+            o.x[16 + 4 * i] = b.x; o.x[16 + 4 * i + 1] = b.y; o.x[16 + 4 * i + 2] = b.z; o.x[16 + 4 * i + 3] = b.w;
+        }
+    } else {
+        const float4 *p = reinterpret_cast<const float4 *>(xs + (size_t)c * E);
+#pragma unroll
+        for (int i = 0; i < E / 4; i++) {
+            float4 a = p[i];
+            o.x[4 * i] = a.x; o.x[4 * i + 1] = a.y; o.x[4 * i + 2] = a.z; o.x[4 * i + 3] = a.w;
+        }
+    }
+    float2 sm = *reinterpret_cast<const float2 *>(sums + 2 * c);
+    o.s_lo = sm.x;
+    o.s_hi = sm.y;
+}
+
+// Sum over the 64 lanes, valid in lane 63.  Four DPP steps inside each row of 16
+// lanes, then the two row broadcasts.
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+#define NH_DPP_ADD(ctrl, rmask)                                                                              \
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, rmask, 0xf, false))
+    NH_DPP_ADD(0xb1, 0xf);   // quad_perm [1,0,3,2]
+    NH_DPP_ADD(0x4e, 0xf);   // quad_perm [2,3,0,1]
+    NH_DPP_ADD(0x141, 0xf);  // row_half_mirror
+    NH_DPP_ADD(0x140, 0xf);  // row_mirror
+    NH_DPP_ADD(0x142, 0xa);  // row_bcast15 into rows 1 and 3
+    NH_DPP_ADD(0x143, 0xc);  // row_bcast31 into rows 2 and 3
+#undef NH_DPP_ADD
+    return v;
+}
+
+template <uint32_t T, int R> struct GemvUnit {
+    Raw<T> raw[R];
+};
+
+template <uint32_t T, int R>
+__global__ __launch_bounds__(GEMV_WAVES * 64, 4) void gemv_kernel(const GemvBatch b) {
     constexpr int E = Geo<T>::E;
     extern __shared__ __align__(16) float lds[];
-    float *xs = lds;                 // x_pad floats
-    float *part = lds + x_pad;       // rw_count * R * kw_count floats
+    float *xs = lds;               // x_pad activations, zero padded
+    float *sums = lds + b.x_pad;   // per chunk: sum of its first half, sum of its second half
 
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    for (uint32_t i = tid; i < x_pad; i += NW * 64) xs[i] = i < m.cols ? x[i] : 0.f;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t n_steps = (b.n_chunks + 63u) / 64u;
+    const uint32_t total_waves = gridDim.x * GEMV_WAVES;
+    const uint32_t cols = b.job[0].m.cols;
+
+    // Unit = (row group g, step s).  State of the unit being fetched:
+    uint32_t g = blockIdx.x * GEMV_WAVES + wave, s = 0;
+
+    auto fetch = [&](uint32_t gg, uint32_t ss, GemvUnit<T, R> &u) {
+        uint32_t j = 0;
+        while (j + 1 < b.n_jobs && gg >= b.job[j + 1].rg_begin) j++;
+        const MatView &m = b.job[j].m;
+        const uint32_t row0 = (gg - b.job[j].rg_begin) * R;
+        uint32_t c = ss * 64u + lane;
+        c = c < b.n_chunks ? c : b.n_chunks - 1;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            uint32_t row = row0 + r < m.rows ? row0 + r : m.rows - 1;
+            load_raw<T>(m, row, c, u.raw[r]);
+        }
+    };
+
+    GemvUnit<T, R> ua, ub;
+    bool have_a = g < b.total_rgs;
+    if (have_a) fetch(g, s, ua);  // in flight while x is staged
+
+    for (uint32_t i = tid; i < b.x_pad; i += GEMV_WAVES * 64) xs[i] = i < cols ? b.x[i] : 0.f;
+    __syncthreads();
+    for (uint32_t c = tid; c < b.n_chunks; c += GEMV_WAVES * 64) {
+        float lo = 0.f, hi = 0.f;
+#pragma unroll
+        for (int i = 0; i < E / 2; i++) {
+            lo += xs[chunk_col<T>(c, i)];
+            hi += xs[chunk_col<T>(c, E / 2 + i)];
+        }
+        sums[2 * c] = lo;
+        sums[2 * c + 1] = hi;
+    }
     __syncthreads();
 
-    const uint32_t kw = wave % kw_count, rw = wave / kw_count;
-    const uint32_t tile_rows = rw_count * R;
-    const uint32_t n_tiles = (m.rows + tile_rows - 1) / tile_rows;
-    const uint32_t n_steps = (n_chunks + 63u) / 64u;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
 
-    for (uint32_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-        const uint32_t row0 = tile * tile_rows + rw * R;
-        float acc[R];
+    auto consume = [&](uint32_t gg, uint32_t ss, const GemvUnit<T, R> &u) {
+        uint32_t c = ss * 64u + lane;
+        const bool active = c < b.n_chunks;
+        c = active ? c : b.n_chunks - 1;
+        XChunk<E> xc;
+        load_x_lds<T>(xs, sums, c, xc);
 #pragma unroll
-        for (int r = 0; r < R; r++) acc[r] = 0.f;
-        if (rw < rw_count && row0 < m.rows) {
-            for (uint32_t s = kw; s < n_steps; s += kw_count) {
-                const uint32_t c = s * 64u + lane;
-                if (c < n_chunks) {
-                    Raw<T> raw[R];
+        for (int r = 0; r < R; r++) {
+            float t = chunk_dot<T>(u.raw[r], xc, c, 0.f);
+            acc[r] += active ? t : 0.f;
+        }
+        if (ss + 1 == n_steps) {  // row group complete
+            uint32_t j = 0;
+            while (j + 1 < b.n_jobs && gg >= b.job[j + 1].rg_begin) j++;
+            const uint32_t row0 = (gg - b.job[j].rg_begin) * R;
+            const uint32_t rows = b.job[j].m.rows;
+            float *y = b.job[j].y;
 #pragma unroll
-                    for (int r = 0; r < R; r++) {
-                        uint32_t row = row0 + r < m.rows ? row0 + r : m.rows - 1;
-                        load_raw<T>(m, row, c, raw[r]);
-                    }
-                    XChunk<E> xc;
-                    load_x<T>(xs, c, xc);
-#pragma unroll
-                    for (int r = 0; r < R; r++) acc[r] = chunk_dot<T>(raw[r], xc, c, acc[r]);
-                }
+            for (int r = 0; r < R; r++) {
+                float tot = wave_sum_dpp(acc[r]);
+                if (lane == 63 && row0 + r < rows) y[row0 + r] = tot;
+                acc[r] = 0.f;
             }
         }
-#pragma unroll
-        for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
-        if (lane == 0 && rw < rw_count) {
-#pragma unroll
-            for (int r = 0; r < R; r++) part[(rw * R + r) * kw_count + kw] = acc[r];
+    };
+    auto advance = [&](uint32_t &gg, uint32_t &ss) {
+        if (ss + 1 < n_steps) {
+            ss++;
+        } else {
+            ss = 0;
+            gg += total_waves;
         }
+    };
+
+    while (have_a) {
+        uint32_t g2 = g, s2 = s;
+        advance(g2, s2);
+        const bool have_b = g2 < b.total_rgs;
+        if (have_b) fetch(g2, s2, ub);
+        consume(g, s, ua);
+        if (!have_b) break;
+        g = g2;
+        s = s2;
+        advance(g, s);
+        have_a = g < b.total_rgs;
+        if (have_a) fetch(g, s, ua);
+        consume(g2, s2, ub);
+    }
+}
+
+// ------------------------------------------------------------------ Q4_K GEMV: one lane per super-block
+//
+// VALU work per weight, not bytes in flight, is what bounds a 4-bit GEMV on this
+// machine (64 non-packed f32 lanes per CU per clock against ~14 weights per CU
+// per clock at full HBM rate), so the Q4_K kernel is laid out to keep that work
+// minimal:
+//   * a lane owns one whole 256-column super-block of one row, so the 16-byte
+//     header is fetched once per 128 code bytes, d/dmin are converted once and
+//     all sixteen 6-bit scale/min extractions use compile-time shifts;
+//   * the code plane is stored piece-major (piece cc of block b at slot
+//     cc * nb + b), so the 64 lanes of a wavefront still read consecutive
+//     16-byte pieces of a row;
+//   * nibbles become floats two at a time through the fp8 (E4M3) unpack: a byte
+//     0x0n read as E4M3 is exactly n * 2^-9 (n < 8 subnormal, 8..15 first binade:
+//     both linear), the factor is folded into d;
+//   * the min term uses the per-sub-block sums of x, computed once per workgroup.
+// LB lanes (a power of two) cover the nb blocks of a row and 64 / LB rows ride in
+// one wavefront step.  Every wavefront streams on its own after the one barrier
+// that publishes x: it keeps the next unit's 144 bytes per lane in flight while it
+// does the arithmetic of the current one.
+
+template <bool FP8> __device__ __forceinline__ float dot4_nib(uint32_t b4, const float *x, float acc) {
+    if constexpr (FP8) {
+        auto lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)b4, false);
+        auto hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)b4, true);
+        acc = fmaf(lo[0], x[0], acc);
+        acc = fmaf(lo[1], x[1], acc);
+        acc = fmaf(hi[0], x[2], acc);
+        acc = fmaf(hi[1], x[3], acc);
+        return acc;
+    } else {
+        return dot4_ub(b4, x, acc);
+    }
+}
+
+template <int LB> __device__ __forceinline__ float group_sum_dpp(float v) {
+#define NH_DPP_ADD(ctrl, rmask)                                                                              \
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, rmask, 0xf, false))
+    if constexpr (LB >= 2) NH_DPP_ADD(0xb1, 0xf);    // quad_perm [1,0,3,2]
+    if constexpr (LB >= 4) NH_DPP_ADD(0x4e, 0xf);    // quad_perm [2,3,0,1]
+    if constexpr (LB >= 8) NH_DPP_ADD(0x141, 0xf);   // row_half_mirror
+    if constexpr (LB >= 16) NH_DPP_ADD(0x140, 0xf);  // row_mirror
+    if constexpr (LB >= 32) NH_DPP_ADD(0x142, 0xa);  // row_bcast15 into rows 1 and 3
+    if constexpr (LB >= 64) NH_DPP_ADD(0x143, 0xc);  // row_bcast31 into rows 2 and 3
+#undef NH_DPP_ADD
+    return v;  // valid in the last lane of every group of LB lanes
+}
+
+#ifdef NH_TRACE
+__device__ unsigned long long nh_trace[8192 * 8];
+#define NH_T(slot) do { if (lane == 0) nh_trace[(size_t)(blockIdx.x * GEMV_WAVES + wave) * 8 + (slot)] = __builtin_readcyclecounter(); } while (0)
+#else
+#define NH_T(slot) do { } while (0)
+#endif
+
+// One unit of work of a lane: header and the eight 16-byte code pieces of its block.
+struct Q4kUnit {
+    uint4 hdr, q[8];
+};
+
+template <int LB, int NW, bool FP8>
+__global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b, const float nib_mul) {
+    constexpr int GEMV_WAVES = NW;  // wavefronts per workgroup of this instantiation
+    constexpr uint32_t RS = 64 / LB;       // rows per wavefront step = rows per row group
+    // LDS row of one (cc, i) slot: LB float4 plus one float4 of padding, so that the 16 slots
+    // consecutive staging lanes write to fall into different banks.
+    constexpr uint32_t XROW = LB * 4 + 4;
+    constexpr uint32_t XS_FLOATS = 64 * XROW;  // x region of one block iteration
+    extern __shared__ __align__(16) float lds[];
+    const uint32_t nb = b.job[0].m.nb, cols = b.job[0].m.cols;
+    const uint32_t n_iter = (nb + LB - 1) / LB;  // block iterations per row (1 unless nb > 64)
+    // x, permuted so that lane blk reads piece i of code piece cc at a compile-time offset:
+    //   float it * XS_FLOATS + (cc*8 + i) * XROW + (blk % LB) * 4 + e,   it = blk / LB
+    float *xs = lds;
+    float *ssum = lds + (size_t)n_iter * XS_FLOATS;  // [it][sub][blk % LB]: sum of x over a sub-block
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t total_waves = gridDim.x * GEMV_WAVES;
+    const uint32_t sub_row = lane / LB, b0 = lane % LB;
+    const uint32_t n_units = b.total_rgs * n_iter;  // unit u = (row group u / n_iter, iteration u % n_iter)
+
+    struct Where {
+        const uint8_t *p0, *p1;
+        float *y;
+        uint32_t s0, s1, rows, row0;
+    };
+    auto locate = [&](uint32_t g) {
+        uint32_t j = 0;
+        while (j + 1 < b.n_jobs && g >= b.job[j + 1].rg_begin) j++;
+        Where w;
+        w.p0 = b.job[j].m.p0;
+        w.p1 = b.job[j].m.p1;
+        w.y = b.job[j].y;
+        w.s0 = b.job[j].m.s0;
+        w.s1 = b.job[j].m.s1;
+        w.rows = b.job[j].m.rows;
+        w.row0 = (g - b.job[j].rg_begin) * RS;
+        return w;
+    };
+    auto fetch = [&](uint32_t u, Q4kUnit &o) {
+        const uint32_t g = u / n_iter, it = u - g * n_iter;
+        const Where w = locate(g);
+        uint32_t row = w.row0 + sub_row;
+        row = row < w.rows ? row : w.rows - 1;
+        uint32_t blk = it * LB + b0;
+        blk = blk < nb ? blk : nb - 1;
+        const uint32_t hoff = row * w.s1 + blk * 16, qoff = row * w.s0 + blk * 16;  // planes stay below 4 GB
+        o.hdr = *reinterpret_cast<const uint4 *>(w.p1 + hoff);
+#pragma unroll
+        for (int cc = 0; cc < 8; cc++) o.q[cc] = *reinterpret_cast<const uint4 *>(w.p0 + (size_t)cc * nb * 16 + qoff);
+    };
+
+    uint32_t u = blockIdx.x * GEMV_WAVES + wave;
+    Q4kUnit ua, ub;
+    NH_T(0);
+    // Stage x once per workgroup; eight consecutive lanes hold one 32-column sub-block.
+    // The x loads are issued before the first unit's weight loads, so they sit at the
+    // head of the memory queue and the weights stream in behind them while x is
+    // being written to LDS.
+    auto stage = [&](uint32_t col, const float4 v) {
+        const uint32_t blk = col >> 8, r = col & 255u, g = r >> 6, r2 = r & 63u, hi = r2 >> 5, r3 = r2 & 31u;
+        const uint32_t cc = 2 * g + (r3 >> 4), t = hi * 16 + (r3 & 15u), it = blk / LB, bl = blk % LB;
+        *reinterpret_cast<float4 *>(xs + (size_t)it * XS_FLOATS + (cc * 8 + (t >> 2)) * XROW + bl * 4) = v;
+        float sm = (v.x + v.y) + (v.z + v.w);
+#define NH_DPP_ADD(ctrl) sm += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), ctrl, 0xf, 0xf, false))
+        NH_DPP_ADD(0xb1);
+        NH_DPP_ADD(0x4e);
+        NH_DPP_ADD(0x141);
+#undef NH_DPP_ADD
+        if ((lane & 7u) == 0) ssum[(it * 8 + (r >> 5)) * LB + bl] = sm;
+    };
+    constexpr int NXV = (LB * 64 + NW * 64 - 1) / (NW * 64);  // float4 per thread for LB blocks of x
+    if (n_iter == 1) {
+        float4 xv[NXV];
+#pragma unroll
+        for (int k = 0; k < NXV; k++) {
+            const uint32_t col = (tid + k * NW * 64) * 4;
+            xv[k] = *reinterpret_cast<const float4 *>(b.x + (col < cols ? col : 0));  // branch-free: stays first
+        }
+        __builtin_amdgcn_sched_barrier(0);  // keep the x loads ahead of the weight loads in the queue
+        fetch(u < n_units ? u : n_units - 1, ua);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < NXV; k++) {
+            const uint32_t col = (tid + k * NW * 64) * 4;
+            if (col < LB * 256) stage(col, col < cols ? xv[k] : make_float4(0.f, 0.f, 0.f, 0.f));
+        }
+        NH_T(1);
         __syncthreads();
-        if (tid < tile_rows) {
-            uint32_t row = tile * tile_rows + tid;
-            if (row < m.rows) {
-                float s = 0.f;
-                for (uint32_t k = 0; k < kw_count; k++) s += part[tid * kw_count + k];
-                y[row] = s;
+        NH_T(2);
+    } else {
+        for (uint32_t col = tid * 4; col < n_iter * LB * 256; col += NW * 64 * 4)
+            stage(col, col < cols ? *reinterpret_cast<const float4 *>(b.x + col) : make_float4(0.f, 0.f, 0.f, 0.f));
+        __syncthreads();
+        if (u < n_units) fetch(u, ua);
+    }
+
+    float acc = 0.f;
+    auto consume = [&](uint32_t uu, const Q4kUnit &q) {
+        const uint32_t g = uu / n_iter, it = uu - g * n_iter;
+        const bool active = it * LB + b0 < nb;
+        const float *xb = xs + (size_t)it * XS_FLOATS + b0 * 4;
+        float t[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) t[k] = 0.f;
+#pragma unroll
+        for (int cc = 0; cc < 8; cc++) {
+            float x[32];
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float4 v = *reinterpret_cast<const float4 *>(xb + (cc * 8 + i) * XROW);
+                x[4 * i] = v.x; x[4 * i + 1] = v.y; x[4 * i + 2] = v.z; x[4 * i + 3] = v.w;
+            }
+            const uint32_t w[4] = {q.q[cc].x, q.q[cc].y, q.q[cc].z, q.q[cc].w};
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                t[cc & ~1] = dot4_nib<FP8>(w[d] & 0x0f0f0f0fu, x + 4 * d, t[cc & ~1]);
+                t[cc | 1] = dot4_nib<FP8>((w[d] >> 4) & 0x0f0f0f0fu, x + 16 + 4 * d, t[cc | 1]);
             }
         }
-        __syncthreads();
+        const uint32_t h1 = q.hdr.y, h2 = q.hdr.z, h3 = q.hdr.w;
+        const float *sp = ssum + (size_t)it * 8 * LB + b0;
+        float S = 0.f, Mn = 0.f;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {  // langtax/src/quant.rs:8901-8912 with constant shifts
+            const float sc_lo = (float)((h1 >> (8 * k)) & 63u), mn_lo = (float)((h2 >> (8 * k)) & 63u);
+            const float sc_hi = (float)(((h3 >> (8 * k)) & 15u) | (((h1 >> (8 * k + 6)) & 3u) << 4));
+            const float mn_hi = (float)(((h3 >> (8 * k + 4)) & 15u) | (((h2 >> (8 * k + 6)) & 3u) << 4));
+            S = fmaf(sc_lo, t[k], S);
+            S = fmaf(sc_hi, t[k + 4], S);
+            Mn = fmaf(mn_lo, sp[k * LB], Mn);
+            Mn = fmaf(mn_hi, sp[(k + 4) * LB], Mn);
+        }
+        const float d = h2f((uint16_t)(q.hdr.x & 0xffffu)) * nib_mul, dmin = h2f((uint16_t)(q.hdr.x >> 16));
+        const float part = fmaf(d, S, -(dmin * Mn));
+        acc += active ? part : 0.f;
+        if (it + 1 == n_iter) {  // row group complete
+            const Where w = locate(g);
+            const float tot = group_sum_dpp<LB>(acc);
+            const uint32_t row = w.row0 + sub_row;
+            if (b0 == LB - 1 && row < w.rows) w.y[row] = tot;
+            acc = 0.f;
+        }
+    };
+
+    while (u < n_units) {
+        const uint32_t u2 = u + total_waves;
+        if (u2 < n_units) fetch(u2, ub);
+#ifdef NH_TRACE
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        NH_T(3);
+#endif
+        consume(u, ua);
+        NH_T(4);
+        if (u2 >= n_units) break;
+        u = u2 + total_waves;
+        if (u < n_units) fetch(u, ua);
+        consume(u2, ub);
     }
 }
 
@@ -525,7 +860,8 @@ template <uint32_t T> __device__ __forceinline__ void dequant8(const MatView &m,
         }
     } else if constexpr (T == T_Q4_K) {
         uint32_t b = k0 >> 8, e = k0 & 255, sub = e >> 5, l = e & 31;
-        uint2 q = *reinterpret_cast<const uint2 *>(m.p0 + ro * m.s0 + (size_t)b * 128 + (sub >> 1) * 32 + l);
+        const uint32_t cc = (sub >> 1) * 2 + (l >> 4);  // 16-byte piece of the block's codes
+        uint2 q = *reinterpret_cast<const uint2 *>(m.p0 + ro * m.s0 + ((size_t)cc * m.nb + b) * 16 + (l & 15));
         uint4 hdr = *reinterpret_cast<const uint4 *>(m.p1 + ro * m.s1 + (size_t)b * 16);
         float d = h2f((uint16_t)(hdr.x & 0xffffu)), dmin = h2f((uint16_t)(hdr.x >> 16));
         float sc, mn;
@@ -634,17 +970,31 @@ void set_device_limits(int cu_count, size_t lds_per_block) {
     if (lds_per_block > 0) g_lds_limit = lds_per_block;
 }
 
-template <uint32_t T, int R, int NW>
-static hipError_t launch_gemv_t(hipStream_t stream, const MatView &m, const float *x, float *y) {
+// Jobs must share x, dtype and column count.  hipErrorInvalidValue = "does not fit this
+// kernel" (x too long for LDS); the caller then uses the tiled kernel.
+template <uint32_t T, int R>
+static hipError_t launch_gemv_t(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n_jobs,
+                                const float *x) {
     constexpr int E = Geo<T>::E;
-    const uint32_t n_chunks = (m.cols + E - 1) / E;
-    const uint32_t n_steps = (n_chunks + 63) / 64;
-    uint32_t kw = n_steps < (uint32_t)NW ? n_steps : (uint32_t)NW;
-    uint32_t rw = NW / kw;
-    const uint32_t x_pad = n_chunks * E;
-    const size_t lds = ((size_t)x_pad + (size_t)rw * R * kw) * sizeof(float);
-    if (lds > g_lds_limit) return hipErrorInvalidValue;  // caller falls back to the tiled kernel
-    auto kern = gemv_kernel<T, R, NW>;
+    GemvBatch b;
+    const uint32_t cols = mats[0].cols;
+    b.n_chunks = (cols + E - 1) / E;
+    b.x_pad = b.n_chunks * E;
+    b.x = x;
+    b.n_jobs = n_jobs;
+    uint32_t rgs = 0;
+    for (uint32_t j = 0; j < n_jobs; j++) {
+        b.job[j].m = mats[j];
+        b.job[j].y = ys[j];
+        b.job[j].rg_begin = rgs;
+        b.job[j].pad = 0;
+        rgs += (mats[j].rows + R - 1) / R;
+    }
+    for (uint32_t j = n_jobs; j < GEMV_MAX_JOBS; j++) b.job[j] = b.job[0];
+    b.total_rgs = rgs;
+    const size_t lds = ((size_t)b.x_pad + 2 * (size_t)b.n_chunks) * sizeof(float);
+    if (lds > g_lds_limit) return hipErrorInvalidValue;
+    auto kern = gemv_kernel<T, R>;
     static size_t configured = 0;  // per instantiation
     if (lds > 48 * 1024 && lds > configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -652,15 +1002,112 @@ static hipError_t launch_gemv_t(hipStream_t stream, const MatView &m, const floa
         if (e != hipSuccess) return e;
         configured = g_lds_limit;
     }
-    const uint32_t tile_rows = rw * R;
-    const uint32_t n_tiles = (m.rows + tile_rows - 1) / tile_rows;
     size_t per_cu = g_lds_limit * 2 / (lds ? lds : 1);  // 160 KB of LDS per CU
     if (per_cu < 1) per_cu = 1;
-    if (per_cu > 4) per_cu = 4;
+    if (per_cu > 2) per_cu = 2;                          // 16 wavefronts per CU
     uint32_t grid = (uint32_t)((size_t)g_cu_count * per_cu);
-    if (grid > n_tiles) grid = n_tiles;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, stream, m, x, y, n_chunks, kw, rw, x_pad);
+    const uint32_t needed = (rgs + GEMV_WAVES - 1) / GEMV_WAVES;
+    if (grid > needed) grid = needed;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(GEMV_WAVES * 64), lds, stream, b);
     return hipGetLastError();
+}
+
+// Decode the sixteen bytes 0x00..0x0f with the fp8 unpack on the device.
+__global__ void fp8_nibble_probe(float *out) {
+    const uint32_t n = threadIdx.x & 15u;
+    auto v = __builtin_amdgcn_cvt_pk_f32_fp8((int)(n | (n << 8) | (n << 16) | (n << 24)), false);
+    auto w = __builtin_amdgcn_cvt_pk_f32_fp8((int)(n | (n << 8) | (n << 16) | (n << 24)), true);
+    out[4 * threadIdx.x] = v[0];
+    out[4 * threadIdx.x + 1] = v[1];
+    out[4 * threadIdx.x + 2] = w[0];
+    out[4 * threadIdx.x + 3] = w[1];
+}
+
+hipError_t probe_fp8_nibble_unit(hipStream_t stream, float *unit_out) {
+    *unit_out = 0.f;
+    float *d = nullptr;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&d), 64 * sizeof(float));
+    if (e != hipSuccess) return e;
+    float h[64];
+    hipLaunchKernelGGL(fp8_nibble_probe, dim3(1), dim3(16), 0, stream, d);
+    e = hipGetLastError();
+    if (e == hipSuccess) e = hipMemcpyAsync(h, d, sizeof h, hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    (void)hipFree(d);
+    if (e != hipSuccess) return e;
+    const float unit = h[4];  // byte 0x01
+    bool linear = unit > 0.f;
+    for (int n = 0; n < 16 && linear; n++)
+        for (int k = 0; k < 4; k++) linear = linear && h[4 * n + k] == (float)n * unit;
+    // the unit must be a power of two so that folding it into a block scale is exact
+    int ex;
+    if (linear && std::frexp(unit, &ex) != 0.5f) linear = false;
+    *unit_out = linear ? unit : 0.f;
+    return hipSuccess;
+}
+
+static float g_nib_mul = 0.f;  // 1 / (value of fp8 byte 0x01); 0 = fp8 unpack not usable
+void set_fp8_nibble_unit(float unit) { g_nib_mul = unit > 0.f ? 1.0f / unit : 0.f; }
+
+template <int LB, int NW>
+static hipError_t launch_q4k_lb(hipStream_t stream, const GemvBatch &b, uint32_t units, size_t lds) {
+    const bool fp8 = g_nib_mul != 0.f;
+    const void *kern = fp8 ? reinterpret_cast<const void *>(gemv_q4k_kernel<LB, NW, true>)
+                           : reinterpret_cast<const void *>(gemv_q4k_kernel<LB, NW, false>);
+    static size_t configured[2] = {0, 0};
+    if (lds > 48 * 1024 && lds > configured[fp8]) {
+        hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g_lds_limit);
+        if (e != hipSuccess) return e;
+        configured[fp8] = g_lds_limit;
+    }
+    size_t per_cu = g_lds_limit * 2 / (lds ? lds : 1);  // 160 KB of LDS per CU
+    if (per_cu < 1) per_cu = 1;
+    if (per_cu > 16 / NW) per_cu = 16 / NW;             // 16 wavefronts per CU
+    uint32_t grid = (uint32_t)((size_t)g_cu_count * per_cu);
+    const uint32_t needed = (units + NW - 1) / NW;
+    if (grid > needed) grid = needed;
+    const float mul = fp8 ? g_nib_mul : 1.0f;
+    if (fp8)
+        hipLaunchKernelGGL((gemv_q4k_kernel<LB, NW, true>), dim3(grid), dim3(NW * 64), lds, stream, b, mul);
+    else
+        hipLaunchKernelGGL((gemv_q4k_kernel<LB, NW, false>), dim3(grid), dim3(NW * 64), lds, stream, b, mul);
+    return hipGetLastError();
+}
+
+static hipError_t launch_gemv_q4k(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n_jobs,
+                                  const float *x) {
+    const uint32_t nb = mats[0].nb;
+    uint32_t lb = 1;
+    while (lb < 64 && lb < nb) lb <<= 1;
+    const uint32_t rg_rows = 64 / lb, n_iter = (nb + lb - 1) / lb;
+    GemvBatch b;
+    b.x = x;
+    b.n_jobs = n_jobs;
+    b.n_chunks = nb * 8;
+    b.x_pad = mats[0].cols;
+    uint32_t rgs = 0;
+    for (uint32_t j = 0; j < n_jobs; j++) {
+        b.job[j].m = mats[j];
+        b.job[j].y = ys[j];
+        b.job[j].rg_begin = rgs;
+        b.job[j].pad = 0;
+        rgs += (mats[j].rows + rg_rows - 1) / rg_rows;
+    }
+    for (uint32_t j = n_jobs; j < GEMV_MAX_JOBS; j++) b.job[j] = b.job[0];
+    b.total_rgs = rgs;
+    const size_t lds = (size_t)n_iter * (64 * (lb * 4 + 4) + lb * 8) * sizeof(float);
+    if (lds > g_lds_limit) return hipErrorInvalidValue;
+    const uint32_t units = rgs * n_iter;
+    switch (lb) {
+    // Short rows: small workgroups, so that even a 1024-row matrix spreads over every CU.
+    case 1: return launch_q4k_lb<1, 4>(stream, b, units, lds);
+    case 2: return launch_q4k_lb<2, 4>(stream, b, units, lds);
+    case 4: return launch_q4k_lb<4, 4>(stream, b, units, lds);
+    case 8: return launch_q4k_lb<8, 4>(stream, b, units, lds);
+    case 16: return launch_q4k_lb<16, 4>(stream, b, units, lds);
+    case 32: return launch_q4k_lb<32, 8>(stream, b, units, lds);
+    default: return launch_q4k_lb<64, 8>(stream, b, units, lds);
+    }
 }
 
 template <uint32_t T>
@@ -673,11 +1120,35 @@ static hipError_t launch_tiled_t(hipStream_t stream, const MatView &m, uint32_t 
 template <uint32_t T>
 static hipError_t launch_t(hipStream_t stream, const MatView &m, uint32_t tokens, const float *x, float *y) {
     if (tokens == 1) {
-        hipError_t e = launch_gemv_t<T, 4, 8>(stream, m, x, y);
+        hipError_t e = T == T_Q4_K ? launch_gemv_q4k(stream, &m, &y, 1, x) : launch_gemv_t<T, 4>(stream, &m, &y, 1, x);
         if (e != hipErrorInvalidValue) return e;
         (void)hipGetLastError();
     }
     return launch_tiled_t<T>(stream, m, tokens, x, y);
+}
+
+template <uint32_t T>
+static hipError_t launch_multi_t(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x) {
+    if constexpr (T == T_Q4_K) return launch_gemv_q4k(stream, mats, ys, n, x);
+    return launch_gemv_t<T, 4>(stream, mats, ys, n, x);
+}
+
+hipError_t launch_gemv_multi(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x) {
+    if (n == 0) return hipSuccess;
+    if (n > GEMV_MAX_JOBS) return hipErrorInvalidValue;
+    for (uint32_t j = 0; j < n; j++)
+        if (mats[j].type != mats[0].type || mats[j].cols != mats[0].cols || mats[j].rows == 0) return hipErrorInvalidValue;
+    switch (mats[0].type) {
+    case T_F32: return launch_multi_t<T_F32>(stream, mats, ys, n, x);
+    case T_F16: return launch_multi_t<T_F16>(stream, mats, ys, n, x);
+    case T_Q4_0: return launch_multi_t<T_Q4_0>(stream, mats, ys, n, x);
+    case T_Q5_0: return launch_multi_t<T_Q5_0>(stream, mats, ys, n, x);
+    case T_Q5_1: return launch_multi_t<T_Q5_1>(stream, mats, ys, n, x);
+    case T_Q8_0: return launch_multi_t<T_Q8_0>(stream, mats, ys, n, x);
+    case T_Q4_K: return launch_multi_t<T_Q4_K>(stream, mats, ys, n, x);
+    case T_Q6_K: return launch_multi_t<T_Q6_K>(stream, mats, ys, n, x);
+    default: return hipErrorInvalidValue;
+    }
 }
 
 hipError_t launch_gemm(hipStream_t stream, const MatView &m, uint32_t tokens, const float *x, float *y) {

@@ -478,3 +478,37 @@ def test_device_pointer_entry_points_match_host_path(pkg, gpu):
         m_host.close()
         m_dev.close()
     stream.destroy()
+
+
+@pytest.mark.parametrize("ty", O.ALL_TYPES, ids=lambda t: O.TYPE_NAMES[t])
+def test_batch_entry_point_fuses_products_that_share_an_input(pkg, gpu, ty):
+    """lnh_gemm_batch_device: products reading the same x (q/k/v, gate/up) go out as one launch;
+    the result must be bit-identical to issuing them one by one."""
+    import importlib
+    hip = importlib.import_module("llama-rust_amd.hiprt")
+    rng = np.random.default_rng(50 + ty)
+    cols = 1024 if K.QK[ty] > 1 else 1000
+    shapes = [(300, cols), (77, cols), (64, cols), (129, 512), (5, cols)]
+    ws = [K.random_packed(ty, r, c, rng) for r, c in shapes]
+    mats = [gpu.upload_packed(ty, r, c, w) for (r, c), w in zip(shapes, ws)]
+    xa = rng.normal(0, 1, cols).astype(np.float32)
+    xb = rng.normal(0, 1, 512).astype(np.float32)
+    xa_d, xb_d = hip.DeviceBuffer.from_numpy(xa), hip.DeviceBuffer.from_numpy(xb)
+    x_ptrs = [xa_d.ptr, xa_d.ptr, xa_d.ptr, xb_d.ptr, xa_d.ptr]   # first three fuse, then two singles
+    ys = [hip.DeviceBuffer(r * 4) for r, _ in shapes]
+    for y in ys:
+        y.fill_byte(0xff)
+    batch = gpu.make_batch(mats, [1] * len(mats), x_ptrs, [y.ptr for y in ys])
+    gpu.gemm_batch_device(batch)
+    gpu.synchronize()
+    for (r, c), w, m, xp, y in zip(shapes, ws, mats, x_ptrs, ys):
+        x = xa if xp == xa_d.ptr else xb
+        got = y.to_numpy(np.float32)
+        check(got, ty, c, 1, r, w, x, f"batch {O.TYPE_NAMES[ty]} {r}x{c}")
+        alone = np.zeros(r, np.float32)
+        gpu.gemv_resident(m, x, alone)
+        assert np.array_equal(got, alone)
+    for b in ys + [xa_d, xb_d]:
+        b.free()
+    for m in mats:
+        m.close()
