@@ -106,6 +106,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="enqueue every product eagerly instead of replaying HIP graphs")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="0 skips the CPU baseline")
     ap.add_argument("--seed", type=int, default=20240531)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB copy kernel three times (known traffic for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         log(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); "
@@ -168,6 +170,14 @@ def main():
         if not np.allclose(got, want, rtol=1e-4, atol=1e-4 * float(np.sqrt(np.mean(want ** 2)))):
             log(f"[bench] FATAL: GPU output of layer-0 {name} disagrees with the CPU oracle")
             return 1
+
+    if args.copy_calibration:
+        src, dst = hip.DeviceBuffer(1 << 30), hip.DeviceBuffer(1 << 30)
+        src.fill_byte(1)
+        for _ in range(3):
+            gpu.calibration_copy(dst.ptr, src.ptr, 1 << 30, stream.ptr)
+        stream.synchronize()
+        src.free(); dst.free()
 
     for _ in range(args.warmup):
         run_layers(); run_head()

@@ -124,6 +124,9 @@ int lnh_gemm_grouped_device(lnh_exec *exec, size_t n_groups, const lnh_matrix *c
  * layer) are issued without a host round trip each. */
 int lnh_gemm_batch_device(lnh_exec *exec, size_t n, const lnh_matrix *const *mats, const size_t *tokens,
                           const float *const *device_x, float *const *device_y, void *stream);
+/* Measurement aid, no counterpart in the reference: a plain device-to-device copy kernel
+ * (nbytes a multiple of 16) whose known traffic calibrates HBM byte counters. */
+int lnh_calibration_copy(lnh_exec *exec, void *device_dst, const void *device_src, size_t nbytes, void *stream);
 /* Block the host until everything enqueued on the executor's own stream is done. */
 int lnh_synchronize(lnh_exec *exec);
 

@@ -89,6 +89,7 @@ def load_library():
         "lnh_gemm_device": (C.c_int, [vp, vp, sz, vp, vp, vp]),
         "lnh_gemm_grouped_device": (C.c_int, [vp, sz, pvp, psz, vp, vp, vp]),
         "lnh_gemm_batch_device": (C.c_int, [vp, sz, pvp, psz, pvp, pvp, vp]),
+        "lnh_calibration_copy": (C.c_int, [vp, vp, vp, sz, vp]),
         "lnh_synchronize": (C.c_int, [vp]),
         "lnh_shape_checked": (C.c_int, [sz, sz, sz, sz, C.POINTER(u32), C.POINTER(u32)]),
         "lnh_validate": (C.c_int, [vp, sz, vp, sz]),
@@ -278,6 +279,10 @@ class HipGemv:
     def gemm_batch_device(self, batch, stream=0):
         n, mats, toks, xs, ys = batch
         self._check(self._lib.lnh_gemm_batch_device(self._h, n, mats, toks, xs, ys, C.c_void_p(stream)))
+
+    def calibration_copy(self, dst_ptr, src_ptr, nbytes, stream=0):
+        self._check(self._lib.lnh_calibration_copy(self._h, C.c_void_p(dst_ptr), C.c_void_p(src_ptr), nbytes,
+                                                   C.c_void_p(stream)))
 
     def synchronize(self):
         self._check(self._lib.lnh_synchronize(self._h))

@@ -458,6 +458,14 @@ int lnh_gemm_batch_device(lnh_exec *e, size_t n, const lnh_matrix *const *mats, 
     return LNH_OK;
 }
 
+int lnh_calibration_copy(lnh_exec *e, void *device_dst, const void *device_src, size_t nbytes, void *stream) {
+    if (!e) return LNH_ERR_INVALID;
+    if (!device_dst || !device_src || nbytes % 16 != 0) return fail(e, LNH_ERR_INVALID, "copy needs device pointers and a multiple of 16 bytes");
+    hipError_t h = nh::launch_copy(stream ? static_cast<hipStream_t>(stream) : e->stream, device_dst, device_src, nbytes);
+    if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
+    return LNH_OK;
+}
+
 int lnh_synchronize(lnh_exec *e) {
     if (!e) return LNH_ERR_INVALID;
     hipError_t h = hipStreamSynchronize(e->stream);

@@ -26,4 +26,7 @@ hipError_t launch_gemm(hipStream_t stream, const MatView &m, uint32_t tokens, co
 // the caller then launches them one by one.
 hipError_t launch_gemv_multi(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x);
 
+// dst[0, nbytes) = src[0, nbytes) (nbytes a multiple of 16): reference traffic for counter calibration.
+hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t nbytes);
+
 }  // namespace nh

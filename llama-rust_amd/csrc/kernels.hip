@@ -1133,6 +1133,17 @@ static hipError_t launch_multi_t(hipStream_t stream, const MatView *mats, float 
     return launch_gemv_t<T, 4>(stream, mats, ys, n, x);
 }
 
+// Plain 16-byte-per-lane copy, used only to calibrate HBM traffic counters.
+__global__ __launch_bounds__(256) void copy_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n16) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
+}
+
+hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t nbytes) {
+    hipLaunchKernelGGL(copy_kernel, dim3(g_cu_count * 8), dim3(256), 0, stream, static_cast<uint4 *>(dst),
+                       static_cast<const uint4 *>(src), nbytes / 16);
+    return hipGetLastError();
+}
+
 hipError_t launch_gemv_multi(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x) {
     if (n == 0) return hipSuccess;
     if (n > GEMV_MAX_JOBS) return hipErrorInvalidValue;
