@@ -130,10 +130,14 @@ __global__ void repack_blocks(MutView v, const uint8_t *__restrict__ src, size_t
     }
     case T_Q6_K: {
         const uint8_t *s = src + r * src_row_bytes + b * 210;
-        uint8_t *ql = v.p0 + r * v.s0 + b * 128;
-        for (int i = 0; i < 128; i++) ql[i] = s[i];
-        uint8_t *qh = v.p1 + r * v.s1 + b * 64;
-        for (int i = 0; i < 64; i++) qh[i] = s[128 + i];
+        for (int cc = 0; cc < 8; cc++) {  // ql: 16-byte piece cc of block b at slot cc * nb + b
+            uint8_t *q = v.p0 + r * v.s0 + ((size_t)cc * v.nb + b) * 16;
+            for (int i = 0; i < 16; i++) q[i] = s[cc * 16 + i];
+        }
+        for (int hc = 0; hc < 4; hc++) {  // qh: 16-byte piece hc of block b at slot hc * nb + b
+            uint8_t *q = v.p1 + r * v.s1 + ((size_t)hc * v.nb + b) * 16;
+            for (int i = 0; i < 16; i++) q[i] = s[128 + hc * 16 + i];
+        }
         uint8_t *sc = v.p2 + r * v.s2 + b * 16;
         for (int i = 0; i < 16; i++) sc[i] = s[192 + i];
         uint8_t *d = v.p3 + r * v.s3 + b * 2;
@@ -288,8 +292,8 @@ template <uint32_t T> __device__ __forceinline__ void load_raw(const MatView &m,
         r.hdr = *reinterpret_cast<const uint4 *>(m.p1 + ro * m.s1 + (size_t)(c >> 3) * 16);
     } else if constexpr (T == T_Q6_K) {
         uint32_t blk = c >> 3, cc = c & 7, n = cc >> 2, k = cc & 1;
-        r.ql = *reinterpret_cast<const uint4 *>(m.p0 + ro * m.s0 + (size_t)c * 16);
-        r.qh = *reinterpret_cast<const uint4 *>(m.p1 + ro * m.s1 + (size_t)blk * 64 + n * 32 + k * 16);
+        r.ql = *reinterpret_cast<const uint4 *>(m.p0 + ro * m.s0 + ((size_t)cc * m.nb + blk) * 16);
+        r.qh = *reinterpret_cast<const uint4 *>(m.p1 + ro * m.s1 + ((size_t)(2 * n + k) * m.nb + blk) * 16);
         r.sc = *reinterpret_cast<const uint2 *>(m.p2 + ro * m.s2 + (size_t)blk * 16 + n * 8);
         r.d = *reinterpret_cast<const uint16_t *>(m.p3 + ro * m.s3 + (size_t)blk * 2);
     }
@@ -799,6 +803,144 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b,
     }
 }
 
+// ------------------------------------------------------------------ Q6_K GEMV: one lane per super-block
+//
+// Same structure as the Q4_K kernel.  A lane owns one 256-column super-block of one
+// row (128 bytes of ql, 64 of qh, 16 int8 scales, d); ql and qh are stored piece-major.
+// Piece cc of ql (n = cc>>2, p = (cc>>1)&1, lh = cc&1) holds in its low nibbles 16
+// codes of quarter p and in its high nibbles 16 codes of quarter p+2 of half n; their
+// two high bits sit in qh piece 2n+lh at bit 2p resp. 2p+4 (langtax/src/quant.rs:8783-8853).
+// The 6-bit codes are assembled four to a register and converted with v_cvt_f32_ubyte;
+// the bias of 32 and the sixteen int8 scales are applied per 16 columns through
+// sum_s sc_s * (sum_k q_k x_k - 32 sum_k x_k).
+
+struct Q6kUnit {
+    uint4 ql[8], qh[4], sc;
+    uint16_t d;
+};
+
+template <int LB, int NW>
+__global__ __launch_bounds__(NW * 64, 4) void gemv_q6k_kernel(const GemvBatch b) {
+    constexpr uint32_t RS = 64 / LB;
+    constexpr uint32_t XROW = LB * 4 + 4;
+    constexpr uint32_t XS_FLOATS = 64 * XROW;
+    extern __shared__ __align__(16) float lds[];
+    const uint32_t nb = b.job[0].m.nb, cols = b.job[0].m.cols;
+    const uint32_t n_iter = (nb + LB - 1) / LB;
+    float *xs = lds;                                  // as in the Q4_K kernel, with this dtype's column order
+    float *ssum = lds + (size_t)n_iter * XS_FLOATS;   // [it][16 column groups][blk % LB]
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t total_waves = gridDim.x * NW;
+    const uint32_t sub_row = lane / LB, b0 = lane % LB;
+    const uint32_t n_units = b.total_rgs * n_iter;
+
+    struct Where {
+        const uint8_t *p0, *p1, *p2, *p3;
+        float *y;
+        uint32_t s0, s1, s2, s3, rows, row0;
+    };
+    auto locate = [&](uint32_t g) {
+        uint32_t j = 0;
+        while (j + 1 < b.n_jobs && g >= b.job[j + 1].rg_begin) j++;
+        Where w;
+        w.p0 = b.job[j].m.p0; w.p1 = b.job[j].m.p1; w.p2 = b.job[j].m.p2; w.p3 = b.job[j].m.p3;
+        w.s0 = b.job[j].m.s0; w.s1 = b.job[j].m.s1; w.s2 = b.job[j].m.s2; w.s3 = b.job[j].m.s3;
+        w.y = b.job[j].y;
+        w.rows = b.job[j].m.rows;
+        w.row0 = (g - b.job[j].rg_begin) * RS;
+        return w;
+    };
+    auto fetch = [&](uint32_t u, Q6kUnit &o) {
+        const uint32_t g = u / n_iter, it = u - g * n_iter;
+        const Where w = locate(g);
+        uint32_t row = w.row0 + sub_row;
+        row = row < w.rows ? row : w.rows - 1;
+        uint32_t blk = it * LB + b0;
+        blk = blk < nb ? blk : nb - 1;
+        const uint8_t *ql = w.p0 + (size_t)row * w.s0 + (size_t)blk * 16;
+        const uint8_t *qh = w.p1 + (size_t)row * w.s1 + (size_t)blk * 16;
+#pragma unroll
+        for (int cc = 0; cc < 8; cc++) o.ql[cc] = *reinterpret_cast<const uint4 *>(ql + (size_t)cc * nb * 16);
+#pragma unroll
+        for (int hc = 0; hc < 4; hc++) o.qh[hc] = *reinterpret_cast<const uint4 *>(qh + (size_t)hc * nb * 16);
+        o.sc = *reinterpret_cast<const uint4 *>(w.p2 + (size_t)row * w.s2 + (size_t)blk * 16);
+        o.d = *reinterpret_cast<const uint16_t *>(w.p3 + (size_t)row * w.s3 + (size_t)blk * 2);
+    };
+
+    // stage x: four consecutive lanes hold one 16-column group
+    auto stage = [&](uint32_t col, const float4 v) {
+        const uint32_t blk = col >> 8, r = col & 255u, n = r >> 7, quarter = (r >> 5) & 3u, l = r & 31u;
+        const uint32_t cc = 4 * n + 2 * (quarter & 1u) + (l >> 4), t = (quarter >> 1) * 16 + (l & 15u);
+        const uint32_t it = blk / LB, bl = blk % LB;
+        *reinterpret_cast<float4 *>(xs + (size_t)it * XS_FLOATS + (cc * 8 + (t >> 2)) * XROW + bl * 4) = v;
+        float sm = (v.x + v.y) + (v.z + v.w);
+        sm += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0xb1, 0xf, 0xf, false));
+        sm += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0x4e, 0xf, 0xf, false));
+        if ((lane & 3u) == 0) ssum[(it * 16 + (r >> 4)) * LB + bl] = sm;
+    };
+    for (uint32_t col = tid * 4; col < n_iter * LB * 256; col += NW * 64 * 4)
+        stage(col, *reinterpret_cast<const float4 *>(b.x + (col < cols ? col : 0)) );
+    __syncthreads();
+
+    float acc = 0.f;
+    Q6kUnit un;
+    for (uint32_t u = blockIdx.x * NW + wave; u < n_units; u += total_waves) {
+        fetch(u, un);
+        const uint32_t g = u / n_iter, it = u - g * n_iter;
+        const bool active = it * LB + b0 < nb;
+        const float *xb = xs + (size_t)it * XS_FLOATS + b0 * 4;
+        float t[16];
+#pragma unroll
+        for (int k = 0; k < 16; k++) t[k] = 0.f;
+#pragma unroll
+        for (int cc = 0; cc < 8; cc++) {
+            constexpr int dummy = 0;
+            (void)dummy;
+            const int n = cc >> 2, p = (cc >> 1) & 1, lh = cc & 1;
+            float x[32];
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float4 v = *reinterpret_cast<const float4 *>(xb + (cc * 8 + i) * XROW);
+                x[4 * i] = v.x; x[4 * i + 1] = v.y; x[4 * i + 2] = v.z; x[4 * i + 3] = v.w;
+            }
+            const uint32_t lo[4] = {un.ql[cc].x, un.ql[cc].y, un.ql[cc].z, un.ql[cc].w};
+            const uint4 hq = un.qh[2 * n + lh];
+            const uint32_t hb[4] = {hq.x, hq.y, hq.z, hq.w};
+            float tl = 0.f, th = 0.f;
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                const uint32_t two_lo = p == 0 ? (hb[d] << 4) : (hb[d] << 2);   // bits 2p..2p+1 moved to 4..5
+                const uint32_t two_hi = p == 0 ? hb[d] : (hb[d] >> 2);          // bits 2p+4..2p+5 moved to 4..5
+                tl = dot4_ub((lo[d] & 0x0f0f0f0fu) | (two_lo & 0x30303030u), x + 4 * d, tl);
+                th = dot4_ub(((lo[d] >> 4) & 0x0f0f0f0fu) | (two_hi & 0x30303030u), x + 16 + 4 * d, th);
+            }
+            t[8 * n + 2 * p + lh] = tl;        // scale index 8n + lh + 2*quarter, quarter = p
+            t[8 * n + 2 * (p + 2) + lh] = th;  // quarter = p + 2
+        }
+        const float *sp = ssum + (size_t)it * 16 * LB + b0;
+        const uint32_t scw[4] = {un.sc.x, un.sc.y, un.sc.z, un.sc.w};
+        float S = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            // t index k = 8n + 2*quarter + lh is also the int8 scale index; the matching 16-column
+            // group of x is (8n + 2*quarter + lh) in column order: group = r >> 4 with r = 128n + 32q + 16lh
+            const float sc = (float)(int)(int8_t)(scw[k >> 2] >> (8 * (k & 3)));
+            S = fmaf(sc, fmaf(-32.f, sp[k * LB], t[k]), S);
+        }
+        const float part = h2f(un.d) * S;
+        acc += active ? part : 0.f;
+        if (it + 1 == n_iter) {
+            const Where w = locate(g);
+            const float tot = group_sum_dpp<LB>(acc);
+            const uint32_t row = w.row0 + sub_row;
+            if (b0 == LB - 1 && row < w.rows) w.y[row] = tot;
+            acc = 0.f;
+        }
+    }
+}
+
 // ------------------------------------------------------------------ tiled GEMM (any token count)
 //
 // Eight consecutive decoded weights of one row starting at column k0 (k0 % 8 == 0).
@@ -876,8 +1018,9 @@ template <uint32_t T> __device__ __forceinline__ void dequant8(const MatView &m,
         }
     } else if constexpr (T == T_Q6_K) {
         uint32_t b = k0 >> 8, e = k0 & 255, n = e >> 7, rr = e & 127, quarter = rr >> 5, l = rr & 31;
-        uint2 lo = *reinterpret_cast<const uint2 *>(m.p0 + ro * m.s0 + (size_t)b * 128 + n * 64 + (quarter & 1) * 32 + l);
-        uint2 hb = *reinterpret_cast<const uint2 *>(m.p1 + ro * m.s1 + (size_t)b * 64 + n * 32 + l);
+        const uint32_t qoff = n * 64 + (quarter & 1) * 32 + l, hoff = n * 32 + l;  // byte offsets inside the block
+        uint2 lo = *reinterpret_cast<const uint2 *>(m.p0 + ro * m.s0 + ((size_t)(qoff >> 4) * m.nb + b) * 16 + (qoff & 15));
+        uint2 hb = *reinterpret_cast<const uint2 *>(m.p1 + ro * m.s1 + ((size_t)(hoff >> 4) * m.nb + b) * 16 + (hoff & 15));
         int8_t s8 = *reinterpret_cast<const int8_t *>(m.p2 + ro * m.s2 + (size_t)b * 16 + n * 8 + quarter * 2 + (l >> 4));
         float ds = h2f(*reinterpret_cast<const uint16_t *>(m.p3 + ro * m.s3 + (size_t)b * 2)) * (float)(int)s8;
         uint32_t nsh = quarter >= 2 ? 4u : 0u, hsh = 2 * quarter;
@@ -1110,6 +1253,61 @@ static hipError_t launch_gemv_q4k(hipStream_t stream, const MatView *mats, float
     }
 }
 
+template <int LB, int NW>
+static hipError_t launch_q6k_lb(hipStream_t stream, const GemvBatch &b, uint32_t units, size_t lds) {
+    auto kern = gemv_q6k_kernel<LB, NW>;
+    static size_t configured = 0;
+    if (lds > 48 * 1024 && lds > configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)g_lds_limit);
+        if (e != hipSuccess) return e;
+        configured = g_lds_limit;
+    }
+    size_t per_cu = g_lds_limit * 2 / (lds ? lds : 1);
+    if (per_cu < 1) per_cu = 1;
+    if (per_cu > 16 / NW) per_cu = 16 / NW;
+    uint32_t grid = (uint32_t)((size_t)g_cu_count * per_cu);
+    const uint32_t needed = (units + NW - 1) / NW;
+    if (grid > needed) grid = needed;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, stream, b);
+    return hipGetLastError();
+}
+
+static hipError_t launch_gemv_q6k(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n_jobs,
+                                  const float *x) {
+    const uint32_t nb = mats[0].nb;
+    uint32_t lb = 1;
+    while (lb < 64 && lb < nb) lb <<= 1;
+    const uint32_t rg_rows = 64 / lb, n_iter = (nb + lb - 1) / lb;
+    GemvBatch b;
+    b.x = x;
+    b.n_jobs = n_jobs;
+    b.n_chunks = nb * 8;
+    b.x_pad = mats[0].cols;
+    uint32_t rgs = 0;
+    for (uint32_t j = 0; j < n_jobs; j++) {
+        b.job[j].m = mats[j];
+        b.job[j].y = ys[j];
+        b.job[j].rg_begin = rgs;
+        b.job[j].pad = 0;
+        rgs += (mats[j].rows + rg_rows - 1) / rg_rows;
+    }
+    for (uint32_t j = n_jobs; j < GEMV_MAX_JOBS; j++) b.job[j] = b.job[0];
+    b.total_rgs = rgs;
+    const size_t lds = (size_t)n_iter * (64 * (lb * 4 + 4) + lb * 16) * sizeof(float);
+    if (lds > g_lds_limit) return hipErrorInvalidValue;
+    const uint32_t units = rgs * n_iter;
+    switch (lb) {
+    case 1: return launch_q6k_lb<1, 4>(stream, b, units, lds);
+    case 2: return launch_q6k_lb<2, 4>(stream, b, units, lds);
+    case 4: return launch_q6k_lb<4, 4>(stream, b, units, lds);
+    case 8: return launch_q6k_lb<8, 4>(stream, b, units, lds);
+    case 16: return launch_q6k_lb<16, 4>(stream, b, units, lds);
+    case 32: return launch_q6k_lb<32, 8>(stream, b, units, lds);
+    default: return launch_q6k_lb<64, 8>(stream, b, units, lds);
+    }
+}
+
 template <uint32_t T>
 static hipError_t launch_tiled_t(hipStream_t stream, const MatView &m, uint32_t tokens, const float *x, float *y) {
     dim3 grid((m.rows + GT_ROWS - 1) / GT_ROWS, (tokens + GT_TOK - 1) / GT_TOK);
@@ -1118,20 +1316,22 @@ static hipError_t launch_tiled_t(hipStream_t stream, const MatView &m, uint32_t 
 }
 
 template <uint32_t T>
+static hipError_t launch_multi_t(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x) {
+    if constexpr (T == T_Q4_K) return launch_gemv_q4k(stream, mats, ys, n, x);
+    if constexpr (T == T_Q6_K) return launch_gemv_q6k(stream, mats, ys, n, x);
+    return launch_gemv_t<T, 4>(stream, mats, ys, n, x);
+}
+
+template <uint32_t T>
 static hipError_t launch_t(hipStream_t stream, const MatView &m, uint32_t tokens, const float *x, float *y) {
     if (tokens == 1) {
-        hipError_t e = T == T_Q4_K ? launch_gemv_q4k(stream, &m, &y, 1, x) : launch_gemv_t<T, 4>(stream, &m, &y, 1, x);
+        hipError_t e = launch_multi_t<T>(stream, &m, &y, 1, x);
         if (e != hipErrorInvalidValue) return e;
         (void)hipGetLastError();
     }
     return launch_tiled_t<T>(stream, m, tokens, x, y);
 }
 
-template <uint32_t T>
-static hipError_t launch_multi_t(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x) {
-    if constexpr (T == T_Q4_K) return launch_gemv_q4k(stream, mats, ys, n, x);
-    return launch_gemv_t<T, 4>(stream, mats, ys, n, x);
-}
 
 // Plain 16-byte-per-lane copy, used only to calibrate HBM traffic counters.
 __global__ __launch_bounds__(256) void copy_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n16) {
