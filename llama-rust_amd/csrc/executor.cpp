@@ -39,6 +39,8 @@ struct lnh_exec {
     hipStream_t stream = nullptr;
     float *d_in = nullptr, *d_out = nullptr;  // device scratch, grow-only
     size_t in_cap = 0, out_cap = 0;           // capacities in floats
+    void *d_ws = nullptr;                     // kernel workspace (multi-token products), grow-only
+    size_t ws_cap = 0;
     std::string err;
 };
 
@@ -104,6 +106,41 @@ int ensure_scratch(lnh_exec *e, size_t in_floats, size_t out_floats) {
         e->in_cap = e->out_cap = 0;
     }
     return LNH_ERR_OOM;
+}
+
+// Workspace of the multi-token kernels.  Work already queued that uses the old
+// buffer is safe: hipFree waits for the device before it releases memory.
+int ensure_workspace(lnh_exec *e, size_t bytes) {
+    if (bytes <= e->ws_cap) return LNH_OK;
+    if (e->d_ws) (void)hipFree(e->d_ws);
+    e->d_ws = nullptr;
+    e->ws_cap = 0;
+    size_t want = bytes + bytes / 4;
+    hipError_t h = hipMalloc(&e->d_ws, want);
+    if (h != hipSuccess) {
+        (void)hipGetLastError();
+        want = bytes;
+        h = hipMalloc(&e->d_ws, want);
+    }
+    if (h != hipSuccess) return hip_fail(e, h, "HIP workspace allocation");
+    e->ws_cap = want;
+    return LNH_OK;
+}
+
+// Launch n products; xs/ys are device pointers.
+int launch_products(lnh_exec *e, hipStream_t s, size_t n, const lnh_matrix *const *mats, const size_t *tokens,
+                    const float *const *xs, float *const *ys) {
+    std::vector<nh::MatView> views(n);
+    std::vector<uint32_t> toks(n);
+    for (size_t g = 0; g < n; g++) {
+        views[g] = mats[g]->view;
+        toks[g] = (uint32_t)tokens[g];
+    }
+    int rc = ensure_workspace(e, nh::gemm_workspace_bytes(views.data(), toks.data(), (uint32_t)n));
+    if (rc != LNH_OK) return rc;
+    hipError_t h = nh::launch_gemm_groups(s, views.data(), toks.data(), xs, ys, (uint32_t)n, e->d_ws, e->ws_cap);
+    if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
+    return LNH_OK;
 }
 
 int make_matrix(lnh_exec *e, uint32_t type, size_t rows, size_t cols, const void *src, bool src_on_device,
@@ -194,16 +231,19 @@ int run_host(lnh_exec *e, size_t n_groups, const lnh_matrix *const *mats, const 
     if (rc != LNH_OK) return rc;
     h = hipMemcpyAsync(e->d_in, x, x_total * sizeof(float), hipMemcpyHostToDevice, e->stream);
     if (h != hipSuccess) return hip_fail(e, h, "HIP input copy");
+    std::vector<const float *> xs(n_groups);
+    std::vector<float *> ys(n_groups);
     size_t xo = 0, yo = 0;
     for (size_t g = 0; g < n_groups; g++) {
-        if (tokens[g] == 0) continue;
-        h = nh::launch_gemm(e->stream, mats[g]->view, (uint32_t)tokens[g], e->d_in + xo, e->d_out + yo);
-        if (h != hipSuccess) {
-            (void)hipStreamSynchronize(e->stream);
-            return hip_fail(e, h, "HIP kernel launch");
-        }
+        xs[g] = e->d_in + xo;
+        ys[g] = e->d_out + yo;
         xo += tokens[g] * mats[g]->view.cols;
         yo += tokens[g] * mats[g]->view.rows;
+    }
+    rc = launch_products(e, e->stream, n_groups, mats, tokens, xs.data(), ys.data());
+    if (rc != LNH_OK) {
+        (void)hipStreamSynchronize(e->stream);
+        return rc;
     }
     h = hipMemcpyAsync(y, e->d_out, y_total * sizeof(float), hipMemcpyDeviceToHost, e->stream);
     hipError_t hs = hipStreamSynchronize(e->stream);
@@ -260,6 +300,7 @@ void lnh_destroy(lnh_exec *e) {
         (void)hipStreamSynchronize(e->stream);
         (void)hipStreamDestroy(e->stream);
     }
+    if (e->d_ws) (void)hipFree(e->d_ws);
     if (e->d_in) (void)hipFree(e->d_in);
     if (e->d_out) (void)hipFree(e->d_out);
     delete e;
@@ -396,9 +437,7 @@ int lnh_gemm_device(lnh_exec *e, const lnh_matrix *m, size_t tokens, const float
     if (rc != LNH_OK) return rc;
     if (!dx || !dy) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
     hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
-    hipError_t h = nh::launch_gemm(s, m->view, (uint32_t)tokens, dx, dy);
-    if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
-    return LNH_OK;
+    return launch_products(e, s, 1, &m, &tokens, &dx, &dy);
 }
 
 int lnh_gemm_grouped_device(lnh_exec *e, size_t n_groups, const lnh_matrix *const *mats, const size_t *tokens,
@@ -409,15 +448,16 @@ int lnh_gemm_grouped_device(lnh_exec *e, size_t n_groups, const lnh_matrix *cons
     if (yt == 0) return LNH_OK;
     if (!dx || !dy) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
     hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
+    std::vector<const float *> xs(n_groups);
+    std::vector<float *> ys(n_groups);
     size_t xo = 0, yo = 0;
     for (size_t g = 0; g < n_groups; g++) {
-        if (tokens[g] == 0) continue;
-        hipError_t h = nh::launch_gemm(s, mats[g]->view, (uint32_t)tokens[g], dx + xo, dy + yo);
-        if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
+        xs[g] = dx + xo;
+        ys[g] = dy + yo;
         xo += tokens[g] * mats[g]->view.cols;
         yo += tokens[g] * mats[g]->view.rows;
     }
-    return LNH_OK;
+    return launch_products(e, s, n_groups, mats, tokens, xs.data(), ys.data());
 }
 
 int lnh_gemm_batch_device(lnh_exec *e, size_t n, const lnh_matrix *const *mats, const size_t *tokens,
@@ -450,7 +490,9 @@ int lnh_gemm_batch_device(lnh_exec *e, size_t n, const lnh_matrix *const *mats, 
         }
         if (h == hipErrorInvalidValue) {
             run = 1;
-            h = nh::launch_gemm(s, mats[i]->view, (uint32_t)tokens[i], dx[i], dy[i]);
+            int rc = launch_products(e, s, 1, &mats[i], &tokens[i], &dx[i], &dy[i]);
+            if (rc != LNH_OK) return rc;
+            h = hipSuccess;
         }
         if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
         i += run;

@@ -12,6 +12,7 @@
 
 #include <cmath>
 #include <cstdlib>
+#include <type_traits>
 
 #include "kernels.h"
 
@@ -1103,6 +1104,335 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(MatView m, const float 
     }
 }
 
+// ------------------------------------------------------------------ MFMA GEMM (two or more tokens)
+//
+// Quantized dtypes only.  A weight is scale * code (+ offset) with an integer code
+// of at most 8 bits, so the code is exact in bf16; an f32 activation is exactly
+// the sum of three bf16 numbers (its 24 significand bits cut into 8 + 8 + 8).
+// Per group of 16 columns that share a scale the kernel therefore forms
+//     P[token, row] = sum_k x[token, k] * code[row, k]
+// with three bf16 MFMAs whose products are exact and whose sums are f32, and
+// then applies the f32 scale (and the offset times the group's sum of x) on the
+// vector ALU:  y += scale * P + offset * Sx.  Nothing is quantized or rounded
+// to fewer than 24 bits anywhere, so the result differs from the reference's
+// (langtax/src/quant.rs:6746-6792, pool.rs:54-101) only in the order of f32 roundings.
+//
+// mm_xsplit_kernel cuts the activations once per call into the MFMA operand
+// layout; gemm_mfma_kernel streams the weights: a workgroup owns 256 rows
+// (one per thread for decoding, 64 per wavefront for the MFMAs) and 32 or 64
+// tokens, walks its share of the columns in steps of 32, and, when the row and
+// token tiles alone would not fill the chip, shares the columns of one tile
+// between several workgroups whose partial sums mm_reduce_kernel adds in a
+// fixed order.
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+constexpr int MM_ROWS = 256;
+constexpr int MM_MAX_JOBS = 8;
+
+struct MmJob {
+    MatView m;
+    const float *x;   // tokens x cols
+    float *y;         // tokens x rows
+    float *part;      // ksplit x tokens x rows when ksplit > 1
+    uint32_t tokens;
+    uint32_t tok_off;    // first token slot of this job in the split activations
+    uint32_t wg_begin;   // first workgroup of this job
+    uint32_t tok_tiles;  // token tiles per row tile
+    uint32_t ksplit;     // workgroups that share the columns of one tile
+    uint32_t pad;
+};
+struct MmBatch {
+    MmJob job[MM_MAX_JOBS];
+    uint4 *xb;   // [group of 16 columns][part 0..2][half 0..1][token slot] x 8 bf16
+    float *sx;   // [group of 16 columns][token slot]: sum of the group's activations
+    uint32_t n_jobs, total_wgs, mpad, any_split;
+};
+
+template <uint32_t T> struct MmTraits { static constexpr bool OFFSET = (T == T_Q4_K || T == T_Q5_1); };
+
+// First of the 16 consecutive columns of group g (0 or 1) of step s.
+template <uint32_t T> __device__ __forceinline__ uint32_t mm_group_col(uint32_t s, uint32_t g) {
+    if constexpr (T == T_Q8_0) return s * 32 + g * 16;
+    else return chunk_col<T>(s, (int)(16 * g));
+}
+
+__device__ __forceinline__ uint32_t bf16_pair(float lo, float hi) {
+    // high halves of the two f32 patterns: exact for integers of at most 8 bits
+    return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+}
+__device__ __forceinline__ uint4 bf16x8_of(const float *f) {
+    return make_uint4(bf16_pair(f[0], f[1]), bf16_pair(f[2], f[3]), bf16_pair(f[4], f[5]), bf16_pair(f[6], f[7]));
+}
+
+template <uint32_t T>
+__global__ __launch_bounds__(256) void mm_xsplit_kernel(const MmBatch b, uint32_t n_groups) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)n_groups * b.mpad) return;
+    const uint32_t gi = (uint32_t)(idx / b.mpad), ts = (uint32_t)(idx % b.mpad);
+    const float *src = nullptr;
+    for (uint32_t j = 0; j < b.n_jobs; j++) {
+        const MmJob &job = b.job[j];
+        if (ts >= job.tok_off && ts - job.tok_off < job.tokens)
+            src = job.x + (size_t)(ts - job.tok_off) * job.m.cols + mm_group_col<T>(gi >> 1, gi & 1u);
+    }
+    float v[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) v[i] = src ? src[i] : 0.f;
+    float sum = 0.f;
+    float hi[16], mid[16], lo[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        sum += v[i];
+        hi[i] = __uint_as_float(__float_as_uint(v[i]) & 0xffff0000u);
+        const float r1 = v[i] - hi[i];  // exact
+        mid[i] = __uint_as_float(__float_as_uint(r1) & 0xffff0000u);
+        lo[i] = r1 - mid[i];            // exact, at most 8 significant bits
+    }
+    const size_t plane = (size_t)2 * b.mpad;  // one part: two halves
+    uint4 *dst = b.xb + (size_t)gi * 3 * plane + ts;
+    dst[0] = bf16x8_of(hi);
+    dst[b.mpad] = bf16x8_of(hi + 8);
+    dst[plane] = bf16x8_of(mid);
+    dst[plane + b.mpad] = bf16x8_of(mid + 8);
+    dst[2 * plane] = bf16x8_of(lo);
+    dst[2 * plane + b.mpad] = bf16x8_of(lo + 8);
+    b.sx[(size_t)gi * b.mpad + ts] = sum;
+}
+
+// Packed bytes of one 32-column step of one row.
+template <uint32_t T> struct MmRaw { Raw<T> r; };
+template <> struct MmRaw<T_Q8_0> { uint4 q0, q1; uint16_t d; };
+
+template <uint32_t T> __device__ __forceinline__ void mm_load(const MatView &m, uint32_t row, uint32_t s, MmRaw<T> &o) {
+    if constexpr (T == T_Q8_0) {
+        const uint4 *q = reinterpret_cast<const uint4 *>(m.p0 + (size_t)row * m.s0 + (size_t)s * 32);
+        o.q0 = q[0];
+        o.q1 = q[1];
+        o.d = *reinterpret_cast<const uint16_t *>(m.p1 + (size_t)row * m.s1 + (size_t)s * 2);
+    } else {
+        load_raw<T>(m, row, s, o.r);
+    }
+}
+
+__device__ __forceinline__ void mm_codes4(uint32_t bytes, float bias, float *f) {
+    f[0] = ub0(bytes) - bias;
+    f[1] = ub1(bytes) - bias;
+    f[2] = ub2(bytes) - bias;
+    f[3] = ub3(bytes) - bias;
+}
+
+// Codes of the two groups of step s as bf16 (frag[g][half]), with scale[g] and
+// offset[g]: W[row, col] = scale * code + offset.
+template <uint32_t T>
+__device__ __forceinline__ void mm_decode(const MmRaw<T> &raw, uint32_t s, uint4 (&frag)[2][2], float (&scale)[2],
+                                          float (&offset)[2]) {
+    float f[2][16];
+    offset[0] = offset[1] = 0.f;
+    if constexpr (T == T_Q8_0) {
+        const uint32_t w[8] = {raw.q0.x, raw.q0.y, raw.q0.z, raw.q0.w, raw.q1.x, raw.q1.y, raw.q1.z, raw.q1.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) f[i >> 2][4 * (i & 3) + k] = sb(w[i], k);
+        scale[0] = scale[1] = h2f(raw.d);
+    } else if constexpr (T == T_Q4_0) {
+        const Raw<T> &r = raw.r;
+        const uint32_t w[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            mm_codes4(w[i] & 0x0f0f0f0fu, 8.f, f[0] + 4 * i);
+            mm_codes4((w[i] >> 4) & 0x0f0f0f0fu, 8.f, f[1] + 4 * i);
+        }
+        scale[0] = scale[1] = h2f(r.d);
+    } else if constexpr (T == T_Q5_0 || T == T_Q5_1) {
+        const Raw<T> &r = raw.r;
+        const uint32_t w[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+        constexpr float bias = T == T_Q5_0 ? 16.f : 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            mm_codes4(q5_bytes(w[i] & 0x0f0f0f0fu, r.qh, 4 * i), bias, f[0] + 4 * i);
+            mm_codes4(q5_bytes((w[i] >> 4) & 0x0f0f0f0fu, r.qh, 16 + 4 * i), bias, f[1] + 4 * i);
+        }
+        if constexpr (T == T_Q5_0) {
+            scale[0] = scale[1] = h2f(r.d);
+        } else {
+            scale[0] = scale[1] = h2f((uint16_t)(r.dm & 0xffffu));
+            offset[0] = offset[1] = h2f((uint16_t)(r.dm >> 16));
+        }
+    } else if constexpr (T == T_Q4_K) {
+        const Raw<T> &r = raw.r;
+        const uint32_t w[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            mm_codes4(w[i] & 0x0f0f0f0fu, 0.f, f[0] + 4 * i);
+            mm_codes4((w[i] >> 4) & 0x0f0f0f0fu, 0.f, f[1] + 4 * i);
+        }
+        const int g = (int)((s & 7u) >> 1);
+        const float d = h2f((uint16_t)(r.hdr.x & 0xffffu)), dmin = h2f((uint16_t)(r.hdr.x >> 16));
+        float sc0, m0, sc1, m1;
+        q4k_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * g, sc0, m0);
+        q4k_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * g + 1, sc1, m1);
+        scale[0] = d * sc0;
+        scale[1] = d * sc1;
+        offset[0] = -(dmin * m0);
+        offset[1] = -(dmin * m1);
+    } else if constexpr (T == T_Q6_K) {
+        const Raw<T> &r = raw.r;
+        const uint32_t lo[4] = {r.ql.x, r.ql.y, r.ql.z, r.ql.w};
+        const uint32_t hb[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
+        const uint32_t cc = s & 7u, h = (cc >> 1) & 1u, k = cc & 1u;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t two_lo = (hb[i] >> (2 * h)) & 0x03030303u;
+            const uint32_t two_hi = (hb[i] >> (2 * h + 4)) & 0x03030303u;
+            mm_codes4((lo[i] & 0x0f0f0f0fu) | (two_lo << 4), 32.f, f[0] + 4 * i);
+            mm_codes4(((lo[i] >> 4) & 0x0f0f0f0fu) | (two_hi << 4), 32.f, f[1] + 4 * i);
+        }
+        const int sh = (int)(8 * (2 * h + k));
+        const float d = h2f(r.d);
+        scale[0] = d * (float)(int)(int8_t)(r.sc.x >> sh);
+        scale[1] = d * (float)(int)(int8_t)(r.sc.y >> sh);
+    }
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+        frag[g][0] = bf16x8_of(f[g]);
+        frag[g][1] = bf16x8_of(f[g] + 8);
+    }
+}
+
+template <uint32_t T, int TT>
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(const MmBatch b) {
+    constexpr bool OFFSET = MmTraits<T>::OFFSET;
+    __shared__ uint4 code_s[2][2][MM_ROWS];   // [group][half of the 16 columns][row]
+    __shared__ float scale_s[2][MM_ROWS];
+    __shared__ float offset_s[OFFSET ? 2 : 1][MM_ROWS];
+    __shared__ float sx_s[OFFSET ? 2 : 1][32 * TT];
+
+    uint32_t j = 0;
+    for (uint32_t k = 1; k < b.n_jobs; k++)
+        if (blockIdx.x >= b.job[k].wg_begin) j = k;
+    const MmJob &job = b.job[j];
+    const MatView &m = job.m;
+    uint32_t local = blockIdx.x - job.wg_begin;
+    const uint32_t ks = local % job.ksplit;
+    local /= job.ksplit;
+    const uint32_t tile_t = local % job.tok_tiles, tile_r = local / job.tok_tiles;
+
+    const uint32_t n_steps = m.cols / 32;
+    const uint32_t s_begin = (uint32_t)((uint64_t)n_steps * ks / job.ksplit);
+    const uint32_t s_end = (uint32_t)((uint64_t)n_steps * (ks + 1) / job.ksplit);
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t n = lane & 31u, kh = lane >> 5;
+    const uint32_t row0 = tile_r * MM_ROWS;
+    const uint32_t drow = row0 + tid < m.rows ? row0 + tid : m.rows - 1;
+    const uint32_t tok0 = tile_t * 32 * TT;          // first token of the tile within the job
+    const uint32_t slot0 = job.tok_off + tok0;       // same, as a slot of the split activations
+    const size_t mpad = b.mpad;
+
+    f32x16 acc[2][TT];
+#pragma unroll
+    for (int rs = 0; rs < 2; rs++)
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[rs][tt][v] = 0.f;
+
+    MmRaw<T> cur;
+    if (s_begin < s_end) mm_load<T>(m, drow, s_begin, cur);
+    for (uint32_t s = s_begin; s < s_end; s++) {
+        {
+            uint4 frag[2][2];
+            float sc[2], of[2];
+            mm_decode<T>(cur, s, frag, sc, of);
+#pragma unroll
+            for (int g = 0; g < 2; g++) {
+                code_s[g][0][tid] = frag[g][0];
+                code_s[g][1][tid] = frag[g][1];
+                scale_s[g][tid] = sc[g];
+                if constexpr (OFFSET) offset_s[g][tid] = of[g];
+            }
+            if constexpr (OFFSET) {
+                if (tid < 2 * 32 * TT) {
+                    const uint32_t g = tid / (32 * TT), i = tid % (32 * TT);
+                    sx_s[g][i] = b.sx[(size_t)(2 * s + g) * mpad + slot0 + i];
+                }
+            }
+        }
+        if (s + 1 < s_end) mm_load<T>(m, drow, s + 1, cur);
+        __syncthreads();
+#pragma unroll
+        for (int g = 0; g < 2; g++) {
+            const size_t gi = (size_t)2 * s + g;
+            bf16x8 wf[2];
+            float sc[2], of[2];
+#pragma unroll
+            for (int rs = 0; rs < 2; rs++) {
+                const uint32_t r = wave * 64 + rs * 32 + n;
+                wf[rs] = __builtin_bit_cast(bf16x8, code_s[g][kh][r]);
+                sc[rs] = scale_s[g][r];
+                of[rs] = OFFSET ? offset_s[g][r] : 0.f;
+            }
+#pragma unroll
+            for (int tt = 0; tt < TT; tt++) {
+                const uint4 *xp = b.xb + (gi * 6 + kh) * mpad + slot0 + tt * 32 + n;
+                const bf16x8 x_hi = __builtin_bit_cast(bf16x8, xp[0]);
+                const bf16x8 x_mid = __builtin_bit_cast(bf16x8, xp[2 * mpad]);
+                const bf16x8 x_lo = __builtin_bit_cast(bf16x8, xp[4 * mpad]);
+                float sxv[16];
+                if constexpr (OFFSET) {
+#pragma unroll
+                    for (int v = 0; v < 16; v++) sxv[v] = sx_s[g][tt * 32 + 8 * (v >> 2) + 4 * kh + (v & 3)];
+                }
+#pragma unroll
+                for (int rs = 0; rs < 2; rs++) {
+                    f32x16 p;
+#pragma unroll
+                    for (int v = 0; v < 16; v++) p[v] = 0.f;
+                    p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_lo, wf[rs], p, 0, 0, 0);
+                    p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_mid, wf[rs], p, 0, 0, 0);
+                    p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_hi, wf[rs], p, 0, 0, 0);
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        acc[rs][tt][v] = fmaf(sc[rs], p[v], acc[rs][tt][v]);
+                        if constexpr (OFFSET) acc[rs][tt][v] = fmaf(of[rs], sxv[v], acc[rs][tt][v]);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    // D[i][j]: lane holds weight row j = lane % 32 and token rows i = 8 (v / 4) + 4 (lane / 32) + v % 4.
+    float *out = job.ksplit > 1 ? job.part + (size_t)ks * job.tokens * m.rows : job.y;
+#pragma unroll
+    for (int rs = 0; rs < 2; rs++) {
+        const uint32_t row = row0 + wave * 64 + rs * 32 + n;
+        if (row >= m.rows) continue;
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const uint32_t t = tok0 + tt * 32 + 8 * (v >> 2) + 4 * kh + (v & 3);
+                if (t < job.tokens) out[(size_t)t * m.rows + row] = acc[rs][tt][v];
+            }
+    }
+}
+
+// y = sum over the column shares, in share order.
+__global__ __launch_bounds__(256) void mm_reduce_kernel(const MmBatch b) {
+    const MmJob &job = b.job[blockIdx.y];
+    const size_t total = (size_t)job.tokens * job.m.rows;
+    if (job.ksplit < 2) return;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        float s = job.part[i];
+        for (uint32_t k = 1; k < job.ksplit; k++) s += job.part[(size_t)k * total + i];
+        job.y[i] = s;
+    }
+}
+
 // ------------------------------------------------------------------ launchers
 
 static int g_cu_count = 256;
@@ -1322,16 +1652,171 @@ static hipError_t launch_multi_t(hipStream_t stream, const MatView *mats, float 
     return launch_gemv_t<T, 4>(stream, mats, ys, n, x);
 }
 
-template <uint32_t T>
-static hipError_t launch_t(hipStream_t stream, const MatView &m, uint32_t tokens, const float *x, float *y) {
-    if (tokens == 1) {
-        hipError_t e = launch_multi_t<T>(stream, &m, &y, 1, x);
-        if (e != hipErrorInvalidValue) return e;
-        (void)hipGetLastError();
+// ---- MFMA GEMM: planning and launch
+
+static bool mm_type(uint32_t type) { return type != T_F32 && type != T_F16 && type_supported(type); }
+
+struct MmPlan {
+    MmBatch b;
+    int tt;             // token tiles of 32 per workgroup (1 or 2)
+    uint32_t n_groups;  // groups of 16 columns
+    size_t xb_bytes, sx_bytes, part_bytes;
+};
+
+static size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// Jobs share dtype and column count; every job has at least two tokens.
+static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *const *xs, float *const *ys, uint32_t n,
+                    MmPlan &p) {
+    MmBatch &b = p.b;
+    uint32_t max_tok = 0, total_tok = 0;
+    for (uint32_t j = 0; j < n; j++) max_tok = tokens[j] > max_tok ? tokens[j] : max_tok;
+    p.tt = max_tok > 32 ? 2 : 1;
+    const uint32_t tile_tok = 32u * (uint32_t)p.tt;
+    uint32_t wgs = 0;
+    bool any_split = false;
+    const uint32_t n_steps = mats[0].cols / 32;
+    for (uint32_t j = 0; j < n; j++) {
+        MmJob &job = b.job[j];
+        job.m = mats[j];
+        job.x = xs ? xs[j] : nullptr;
+        job.y = ys ? ys[j] : nullptr;
+        job.part = nullptr;
+        job.tokens = tokens[j];
+        job.tok_off = total_tok;
+        job.wg_begin = wgs;
+        job.tok_tiles = (tokens[j] + tile_tok - 1) / tile_tok;
+        // The column split of a product depends on that product alone, so that its
+        // result does not change with what else shares the launch.
+        const uint32_t tiles = job.tok_tiles * ((mats[j].rows + MM_ROWS - 1) / MM_ROWS);
+        uint32_t ks = (uint32_t)g_cu_count / tiles;
+        if (ks > n_steps / 4) ks = n_steps / 4;
+        if (ks > 16) ks = 16;
+        if (ks < 1) ks = 1;
+        job.ksplit = ks;
+        job.pad = 0;
+        wgs += tiles * ks;
+        any_split = any_split || ks > 1;
+        total_tok += tokens[j];
     }
-    return launch_tiled_t<T>(stream, m, tokens, x, y);
+    for (uint32_t j = n; j < MM_MAX_JOBS; j++) b.job[j] = b.job[0];
+    b.n_jobs = n;
+    b.mpad = total_tok + 64;  // a tile may read up to 63 slots past its job's last token
+    b.total_wgs = wgs;
+    b.any_split = any_split ? 1u : 0u;
+    p.n_groups = mats[0].cols / 16;
+    p.xb_bytes = up256((size_t)p.n_groups * 6 * b.mpad * sizeof(uint4));
+    p.sx_bytes = up256((size_t)p.n_groups * b.mpad * sizeof(float));
+    size_t part = 0;
+    for (uint32_t j = 0; j < n; j++)
+        if (b.job[j].ksplit > 1) part += up256((size_t)b.job[j].ksplit * tokens[j] * mats[j].rows * sizeof(float));
+    p.part_bytes = part;
 }
 
+template <uint32_t T>
+static hipError_t launch_mm_t(hipStream_t stream, MmPlan &p, void *ws, size_t ws_bytes) {
+    if (p.xb_bytes + p.sx_bytes + p.part_bytes > ws_bytes) return hipErrorInvalidValue;
+    MmBatch &b = p.b;
+    uint8_t *base = static_cast<uint8_t *>(ws);
+    b.xb = reinterpret_cast<uint4 *>(base);
+    b.sx = reinterpret_cast<float *>(base + p.xb_bytes);
+    uint8_t *part = base + p.xb_bytes + p.sx_bytes;
+    for (uint32_t j = 0; j < b.n_jobs; j++)
+        if (b.job[j].ksplit > 1) {
+            b.job[j].part = reinterpret_cast<float *>(part);
+            part += up256((size_t)b.job[j].ksplit * b.job[j].tokens * b.job[j].m.rows * sizeof(float));
+        }
+    const size_t split_threads = (size_t)p.n_groups * b.mpad;
+    hipLaunchKernelGGL(mm_xsplit_kernel<T>, dim3((unsigned)((split_threads + 255) / 256)), dim3(256), 0, stream, b,
+                       p.n_groups);
+    if (p.tt == 1)
+        hipLaunchKernelGGL((gemm_mfma_kernel<T, 1>), dim3(b.total_wgs), dim3(256), 0, stream, b);
+    else
+        hipLaunchKernelGGL((gemm_mfma_kernel<T, 2>), dim3(b.total_wgs), dim3(256), 0, stream, b);
+    if (b.any_split) hipLaunchKernelGGL(mm_reduce_kernel, dim3(64, b.n_jobs), dim3(256), 0, stream, b);
+    return hipGetLastError();
+}
+
+static hipError_t launch_mm(hipStream_t stream, MmPlan &p, void *ws, size_t ws_bytes) {
+    switch (p.b.job[0].m.type) {
+    case T_Q4_0: return launch_mm_t<T_Q4_0>(stream, p, ws, ws_bytes);
+    case T_Q5_0: return launch_mm_t<T_Q5_0>(stream, p, ws, ws_bytes);
+    case T_Q5_1: return launch_mm_t<T_Q5_1>(stream, p, ws, ws_bytes);
+    case T_Q8_0: return launch_mm_t<T_Q8_0>(stream, p, ws, ws_bytes);
+    case T_Q4_K: return launch_mm_t<T_Q4_K>(stream, p, ws, ws_bytes);
+    case T_Q6_K: return launch_mm_t<T_Q6_K>(stream, p, ws, ws_bytes);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+// Single-token products, and F32/F16 products of any token count.
+static hipError_t launch_plain(hipStream_t stream, const MatView &m, uint32_t tokens, const float *x, float *y) {
+    auto run = [&](auto tag) -> hipError_t {
+        constexpr uint32_t T = decltype(tag)::value;
+        if (tokens == 1) {
+            hipError_t e = launch_multi_t<T>(stream, &m, &y, 1, x);
+            if (e != hipErrorInvalidValue) return e;
+            (void)hipGetLastError();
+        }
+        return launch_tiled_t<T>(stream, m, tokens, x, y);
+    };
+    switch (m.type) {
+    case T_F32: return run(std::integral_constant<uint32_t, T_F32>{});
+    case T_F16: return run(std::integral_constant<uint32_t, T_F16>{});
+    case T_Q4_0: return run(std::integral_constant<uint32_t, T_Q4_0>{});
+    case T_Q5_0: return run(std::integral_constant<uint32_t, T_Q5_0>{});
+    case T_Q5_1: return run(std::integral_constant<uint32_t, T_Q5_1>{});
+    case T_Q8_0: return run(std::integral_constant<uint32_t, T_Q8_0>{});
+    case T_Q4_K: return run(std::integral_constant<uint32_t, T_Q4_K>{});
+    case T_Q6_K: return run(std::integral_constant<uint32_t, T_Q6_K>{});
+    default: return hipErrorInvalidValue;
+    }
+}
+
+// Length of the run of groups starting at g that one MFMA launch can take.
+static uint32_t mm_run(const MatView *mats, const uint32_t *tokens, uint32_t n, uint32_t g) {
+    if (!mm_type(mats[g].type) || tokens[g] < 2) return 0;
+    uint32_t run = 1;
+    while (g + run < n && run < (uint32_t)MM_MAX_JOBS && tokens[g + run] >= 2 && mats[g + run].type == mats[g].type &&
+           mats[g + run].cols == mats[g].cols)
+        run++;
+    return run;
+}
+
+size_t gemm_workspace_bytes(const MatView *mats, const uint32_t *tokens, uint32_t n) {
+    size_t need = 0;
+    for (uint32_t g = 0; g < n;) {
+        if (tokens[g] == 0 || mats[g].rows == 0) { g++; continue; }
+        const uint32_t run = mm_run(mats, tokens, n, g);
+        if (run == 0) { g++; continue; }
+        MmPlan p;
+        mm_plan(mats + g, tokens + g, nullptr, nullptr, run, p);
+        const size_t bytes = p.xb_bytes + p.sx_bytes + p.part_bytes;
+        need = bytes > need ? bytes : need;
+        g += run;
+    }
+    return need;
+}
+
+hipError_t launch_gemm_groups(hipStream_t stream, const MatView *mats, const uint32_t *tokens, const float *const *xs,
+                              float *const *ys, uint32_t n, void *ws, size_t ws_bytes) {
+    for (uint32_t g = 0; g < n;) {
+        if (tokens[g] == 0 || mats[g].rows == 0) { g++; continue; }
+        const uint32_t run = mm_run(mats, tokens, n, g);
+        hipError_t e;
+        if (run == 0) {
+            e = launch_plain(stream, mats[g], tokens[g], xs[g], ys[g]);
+            g++;
+        } else {
+            MmPlan p;
+            mm_plan(mats + g, tokens + g, xs + g, ys + g, run, p);
+            e = launch_mm(stream, p, ws, ws_bytes);
+            g += run;
+        }
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
 
 // Plain 16-byte-per-lane copy, used only to calibrate HBM traffic counters.
 __global__ __launch_bounds__(256) void copy_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n16) {
@@ -1362,19 +1847,9 @@ hipError_t launch_gemv_multi(hipStream_t stream, const MatView *mats, float *con
     }
 }
 
-hipError_t launch_gemm(hipStream_t stream, const MatView &m, uint32_t tokens, const float *x, float *y) {
-    if (m.rows == 0 || tokens == 0) return hipSuccess;
-    switch (m.type) {
-    case T_F32: return launch_t<T_F32>(stream, m, tokens, x, y);
-    case T_F16: return launch_t<T_F16>(stream, m, tokens, x, y);
-    case T_Q4_0: return launch_t<T_Q4_0>(stream, m, tokens, x, y);
-    case T_Q5_0: return launch_t<T_Q5_0>(stream, m, tokens, x, y);
-    case T_Q5_1: return launch_t<T_Q5_1>(stream, m, tokens, x, y);
-    case T_Q8_0: return launch_t<T_Q8_0>(stream, m, tokens, x, y);
-    case T_Q4_K: return launch_t<T_Q4_K>(stream, m, tokens, x, y);
-    case T_Q6_K: return launch_t<T_Q6_K>(stream, m, tokens, x, y);
-    default: return hipErrorInvalidValue;
-    }
+hipError_t launch_gemm(hipStream_t stream, const MatView &m, uint32_t tokens, const float *x, float *y, void *ws,
+                       size_t ws_bytes) {
+    return launch_gemm_groups(stream, &m, &tokens, &x, &y, 1, ws, ws_bytes);
 }
 
 }  // namespace nh
