@@ -31,7 +31,8 @@ struct lnh_matrix {
     std::shared_ptr<Ctx> ctx;
     void *dev = nullptr;
     size_t dev_bytes = 0;
-    nh::MatView view{};
+    nh::MatView view{};   // planes the single-token kernels read
+    nh::MatView tiled{};  // row-interleaved copy the multi-token kernels read (quantized dtypes)
 };
 
 struct lnh_exec {
@@ -130,15 +131,16 @@ int ensure_workspace(lnh_exec *e, size_t bytes) {
 // Launch n products; xs/ys are device pointers.
 int launch_products(lnh_exec *e, hipStream_t s, size_t n, const lnh_matrix *const *mats, const size_t *tokens,
                     const float *const *xs, float *const *ys) {
-    std::vector<nh::MatView> views(n);
+    std::vector<nh::MatView> views(n), tiled(n);
     std::vector<uint32_t> toks(n);
     for (size_t g = 0; g < n; g++) {
         views[g] = mats[g]->view;
+        tiled[g] = mats[g]->tiled;
         toks[g] = (uint32_t)tokens[g];
     }
     int rc = ensure_workspace(e, nh::gemm_workspace_bytes(views.data(), toks.data(), (uint32_t)n));
     if (rc != LNH_OK) return rc;
-    hipError_t h = nh::launch_gemm_groups(s, views.data(), toks.data(), xs, ys, (uint32_t)n, e->d_ws, e->ws_cap);
+    hipError_t h = nh::launch_gemm_groups(s, views.data(), tiled.data(), toks.data(), xs, ys, (uint32_t)n, e->d_ws, e->ws_cap);
     if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
     return LNH_OK;
 }
@@ -146,10 +148,11 @@ int launch_products(lnh_exec *e, hipStream_t s, size_t n, const lnh_matrix *cons
 int make_matrix(lnh_exec *e, uint32_t type, size_t rows, size_t cols, const void *src, bool src_on_device,
                 size_t nbytes, lnh_matrix **out) {
     nh::PlaneSpec ps = nh::plane_spec(type, rows, cols);
+    nh::TiledSpec ts = nh::tiled_spec(type, rows, cols);
     hipError_t h = hipSetDevice(e->ctx->device);
     if (h != hipSuccess) return hip_fail(e, h, "hipSetDevice");
     void *dev = nullptr;
-    h = hipMalloc(&dev, ps.total);
+    h = hipMalloc(&dev, ps.total + ts.total);
     if (h != hipSuccess) return hip_fail(e, h, "HIP matrix allocation");
     void *staging = nullptr;
     const void *src_dev = src;
@@ -165,7 +168,7 @@ int make_matrix(lnh_exec *e, uint32_t type, size_t rows, size_t cols, const void
     auto m = std::make_unique<lnh_matrix>();
     m->ctx = e->ctx;
     m->dev = dev;
-    m->dev_bytes = ps.total;
+    m->dev_bytes = ps.total + ts.total;
     uint8_t *base = static_cast<uint8_t *>(dev);
     m->view.p0 = base + ps.offset[0];
     m->view.p1 = base + ps.offset[1];
@@ -179,6 +182,21 @@ int make_matrix(lnh_exec *e, uint32_t type, size_t rows, size_t cols, const void
     m->view.rows = (uint32_t)rows;
     m->view.cols = (uint32_t)cols;
     m->view.nb = (uint32_t)(cols / nh::block_elems(type));
+    if (ts.total != 0) {
+        uint8_t *tb = base + ps.total;
+        m->tiled = m->view;
+        m->tiled.p0 = tb + ts.offset[0];
+        m->tiled.p1 = tb + ts.offset[1];
+        m->tiled.p2 = tb + ts.offset[2];
+        m->tiled.p3 = tb + ts.offset[3];
+        m->tiled.s0 = (uint32_t)ts.per_row[0];
+        m->tiled.s1 = (uint32_t)ts.per_row[1];
+        m->tiled.s2 = (uint32_t)ts.per_row[2];
+        m->tiled.s3 = (uint32_t)ts.per_row[3];
+        // rows that pad the last tile are decoded like any other and then dropped: give them defined bytes
+        if (h == hipSuccess) h = hipMemsetAsync(tb, 0, ts.total, e->stream);
+        if (h == hipSuccess) h = nh::launch_repack_tiled(e->stream, m->tiled, src_dev);
+    }
     if (h == hipSuccess) h = nh::launch_repack(e->stream, m->view, src_dev);
     hipError_t hs = hipStreamSynchronize(e->stream);
     if (h == hipSuccess) h = hs;

@@ -17,19 +17,21 @@ hipError_t probe_fp8_nibble_unit(hipStream_t stream, float *unit_out);
 
 // Scatter the GGUF bytes at src_device (device memory) into the planes of m.
 hipError_t launch_repack(hipStream_t stream, const MatView &m, const void *src_device);
+// Same for the tiled copy (matview.h); tiled.s0..s3 hold the units per row of each plane.
+hipError_t launch_repack_tiled(hipStream_t stream, const MatView &tiled, const void *src_device);
 
 // y[t, r] = sum_c W[r, c] x[t, c]; x and y are device pointers, token-major.
-// Products of two or more tokens by a quantized matrix run on the matrix cores
-// and need device workspace: ws must hold gemm_workspace_bytes() for the same
+// Products of two or more tokens by a quantized matrix run on the matrix cores,
+// read the tiled copy of the matrix and need device workspace: ws must hold gemm_workspace_bytes() for the same
 // arguments (hipErrorInvalidValue otherwise).  The workspace is only used by
 // work queued on `stream`, so calls on one stream may share it.
 size_t gemm_workspace_bytes(const MatView *mats, const uint32_t *tokens, uint32_t n);
-hipError_t launch_gemm(hipStream_t stream, const MatView &m, uint32_t tokens, const float *x, float *y, void *ws,
-                       size_t ws_bytes);
+hipError_t launch_gemm(hipStream_t stream, const MatView &m, const MatView &tiled, uint32_t tokens, const float *x,
+                       float *y, void *ws, size_t ws_bytes);
 // n independent products (the experts of one MoE projection, say): consecutive
 // groups of equal dtype and column count share launches, up to 8 per launch.
-hipError_t launch_gemm_groups(hipStream_t stream, const MatView *mats, const uint32_t *tokens, const float *const *xs,
-                              float *const *ys, uint32_t n, void *ws, size_t ws_bytes);
+hipError_t launch_gemm_groups(hipStream_t stream, const MatView *mats, const MatView *tiled, const uint32_t *tokens,
+                              const float *const *xs, float *const *ys, uint32_t n, void *ws, size_t ws_bytes);
 
 // One launch for up to 8 single-token products that read the same x and share dtype
 // and column count (q/k/v, gate/up).  hipErrorInvalidValue = not fusable this way;

@@ -159,6 +159,65 @@ __global__ void repack_plain(uint8_t *dst, size_t dst_stride, const uint8_t *__r
     dst[idx] = c < row_bytes ? src[r * row_bytes + c] : (uint8_t)0;
 }
 
+// Tiled copy (matview.h): one thread per GGUF block.  In the MutView of a tiled
+// copy s0..s3 hold the units per row of each plane.
+__global__ void repack_blocks_tiled(MutView v, const uint8_t *__restrict__ src, size_t src_row_bytes) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t total = (size_t)v.rows * v.nb;
+    if (idx >= total) return;
+    const size_t r = idx / v.nb, b = idx % v.nb, tile = r / TILE_ROWS, rr = r % TILE_ROWS;
+    auto unit = [&](uint8_t *p, uint32_t per_row, size_t i, size_t bytes) {
+        return p + ((tile * per_row + i) * TILE_ROWS + rr) * bytes;
+    };
+    auto copy = [](uint8_t *d, const uint8_t *s, int n) {
+        for (int i = 0; i < n; i++) d[i] = s[i];
+    };
+    switch (v.type) {
+    case T_Q8_0: {
+        const uint8_t *s = src + r * src_row_bytes + b * 34;
+        copy(unit(v.p1, v.s1, b, 2), s, 2);
+        copy(unit(v.p0, v.s0, 2 * b, 16), s + 2, 16);
+        copy(unit(v.p0, v.s0, 2 * b + 1, 16), s + 18, 16);
+        break;
+    }
+    case T_Q4_0: {
+        const uint8_t *s = src + r * src_row_bytes + b * 18;
+        copy(unit(v.p1, v.s1, b, 2), s, 2);
+        copy(unit(v.p0, v.s0, b, 16), s + 2, 16);
+        break;
+    }
+    case T_Q5_0: {
+        const uint8_t *s = src + r * src_row_bytes + b * 22;
+        copy(unit(v.p2, v.s2, b, 2), s, 2);
+        copy(unit(v.p1, v.s1, b, 4), s + 2, 4);
+        copy(unit(v.p0, v.s0, b, 16), s + 6, 16);
+        break;
+    }
+    case T_Q5_1: {
+        const uint8_t *s = src + r * src_row_bytes + b * 24;
+        copy(unit(v.p2, v.s2, b, 4), s, 4);
+        copy(unit(v.p1, v.s1, b, 4), s + 4, 4);
+        copy(unit(v.p0, v.s0, b, 16), s + 8, 16);
+        break;
+    }
+    case T_Q4_K: {
+        const uint8_t *s = src + r * src_row_bytes + b * 144;
+        copy(unit(v.p1, v.s1, b, 16), s, 16);
+        for (int cc = 0; cc < 8; cc++) copy(unit(v.p0, v.s0, 8 * b + cc, 16), s + 16 + 16 * cc, 16);
+        break;
+    }
+    case T_Q6_K: {
+        const uint8_t *s = src + r * src_row_bytes + b * 210;
+        for (int cc = 0; cc < 8; cc++) copy(unit(v.p0, v.s0, 8 * b + cc, 16), s + 16 * cc, 16);
+        for (int hc = 0; hc < 4; hc++) copy(unit(v.p1, v.s1, 4 * b + hc, 16), s + 128 + 16 * hc, 16);
+        for (int n = 0; n < 2; n++) copy(unit(v.p2, v.s2, 2 * b + n, 8), s + 192 + 8 * n, 8);
+        copy(unit(v.p3, v.s3, b, 2), s + 208, 2);
+        break;
+    }
+    default: break;
+    }
+}
+
 static MutView mut_view(const MatView &m) {
     MutView v;
     v.p0 = const_cast<uint8_t *>(m.p0);
@@ -168,6 +227,14 @@ static MutView mut_view(const MatView &m) {
     v.s0 = m.s0; v.s1 = m.s1; v.s2 = m.s2; v.s3 = m.s3;
     v.type = m.type; v.rows = m.rows; v.cols = m.cols; v.nb = m.nb;
     return v;
+}
+
+hipError_t launch_repack_tiled(hipStream_t stream, const MatView &tiled, const void *src_device) {
+    if (tiled.rows == 0 || tiled.p0 == nullptr) return hipSuccess;
+    size_t total = (size_t)tiled.rows * tiled.nb;
+    hipLaunchKernelGGL(repack_blocks_tiled, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, mut_view(tiled),
+                       static_cast<const uint8_t *>(src_device), gguf_row_bytes(tiled.type, tiled.cols));
+    return hipGetLastError();
 }
 
 hipError_t launch_repack(hipStream_t stream, const MatView &m, const void *src_device) {
@@ -1128,11 +1195,11 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(MatView m, const float 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
-constexpr int MM_ROWS = 256;
+constexpr int MM_ROWS = TILE_ROWS;  // rows per workgroup = row tile of the tiled copy
 constexpr int MM_MAX_JOBS = 8;
 
 struct MmJob {
-    MatView m;
+    MatView m;        // the tiled copy (matview.h)
     const float *x;   // tokens x cols
     float *y;         // tokens x rows
     float *part;      // ksplit x tokens x rows when ksplit > 1
@@ -1150,7 +1217,10 @@ struct MmBatch {
     uint32_t n_jobs, total_wgs, mpad, any_split;
 };
 
-template <uint32_t T> struct MmTraits { static constexpr bool OFFSET = (T == T_Q4_K || T == T_Q5_1); };
+template <uint32_t T> struct MmTraits {
+    static constexpr bool OFFSET = (T == T_Q4_K || T == T_Q5_1);                       // W = scale * code + offset
+    static constexpr bool SAME_SCALE = (T == T_Q4_0 || T == T_Q5_0 || T == T_Q5_1 || T == T_Q8_0);  // per 32 columns
+};
 
 // First of the 16 consecutive columns of group g (0 or 1) of step s.
 template <uint32_t T> __device__ __forceinline__ uint32_t mm_group_col(uint32_t s, uint32_t g) {
@@ -1205,14 +1275,37 @@ __global__ __launch_bounds__(256) void mm_xsplit_kernel(const MmBatch b, uint32_
 template <uint32_t T> struct MmRaw { Raw<T> r; };
 template <> struct MmRaw<T_Q8_0> { uint4 q0, q1; uint16_t d; };
 
-template <uint32_t T> __device__ __forceinline__ void mm_load(const MatView &m, uint32_t row, uint32_t s, MmRaw<T> &o) {
+// Step s of the row that thread `tid` of row tile `tile` decodes, from the tiled copy g
+// (g.s0..s3 = units per row of each plane).
+template <uint32_t T>
+__device__ __forceinline__ void mm_load(const MatView &g, uint32_t tile, uint32_t tid, uint32_t s, MmRaw<T> &o) {
+    auto at = [&](const uint8_t *p, uint32_t per_row, size_t i, size_t bytes) {
+        return p + (((size_t)tile * per_row + i) * TILE_ROWS + tid) * bytes;
+    };
     if constexpr (T == T_Q8_0) {
-        const uint4 *q = reinterpret_cast<const uint4 *>(m.p0 + (size_t)row * m.s0 + (size_t)s * 32);
-        o.q0 = q[0];
-        o.q1 = q[1];
-        o.d = *reinterpret_cast<const uint16_t *>(m.p1 + (size_t)row * m.s1 + (size_t)s * 2);
-    } else {
-        load_raw<T>(m, row, s, o.r);
+        o.q0 = *reinterpret_cast<const uint4 *>(at(g.p0, g.s0, 2 * (size_t)s, 16));
+        o.q1 = *reinterpret_cast<const uint4 *>(at(g.p0, g.s0, 2 * (size_t)s + 1, 16));
+        o.d = *reinterpret_cast<const uint16_t *>(at(g.p1, g.s1, s, 2));
+    } else if constexpr (T == T_Q4_0) {
+        o.r.q = *reinterpret_cast<const uint4 *>(at(g.p0, g.s0, s, 16));
+        o.r.d = *reinterpret_cast<const uint16_t *>(at(g.p1, g.s1, s, 2));
+    } else if constexpr (T == T_Q5_0) {
+        o.r.q = *reinterpret_cast<const uint4 *>(at(g.p0, g.s0, s, 16));
+        o.r.qh = *reinterpret_cast<const uint32_t *>(at(g.p1, g.s1, s, 4));
+        o.r.d = *reinterpret_cast<const uint16_t *>(at(g.p2, g.s2, s, 2));
+    } else if constexpr (T == T_Q5_1) {
+        o.r.q = *reinterpret_cast<const uint4 *>(at(g.p0, g.s0, s, 16));
+        o.r.qh = *reinterpret_cast<const uint32_t *>(at(g.p1, g.s1, s, 4));
+        o.r.dm = *reinterpret_cast<const uint32_t *>(at(g.p2, g.s2, s, 4));
+    } else if constexpr (T == T_Q4_K) {
+        o.r.q = *reinterpret_cast<const uint4 *>(at(g.p0, g.s0, s, 16));
+        o.r.hdr = *reinterpret_cast<const uint4 *>(at(g.p1, g.s1, s >> 3, 16));
+    } else if constexpr (T == T_Q6_K) {
+        const uint32_t blk = s >> 3, cc = s & 7u, n = cc >> 2, k = cc & 1u;
+        o.r.ql = *reinterpret_cast<const uint4 *>(at(g.p0, g.s0, s, 16));
+        o.r.qh = *reinterpret_cast<const uint4 *>(at(g.p1, g.s1, (size_t)blk * 4 + 2 * n + k, 16));
+        o.r.sc = *reinterpret_cast<const uint2 *>(at(g.p2, g.s2, (size_t)blk * 2 + n, 8));
+        o.r.d = *reinterpret_cast<const uint16_t *>(at(g.p3, g.s3, blk, 2));
     }
 }
 
@@ -1269,11 +1362,18 @@ __device__ __forceinline__ void mm_decode(const MmRaw<T> &raw, uint32_t s, uint4
             mm_codes4(w[i] & 0x0f0f0f0fu, 0.f, f[0] + 4 * i);
             mm_codes4((w[i] >> 4) & 0x0f0f0f0fu, 0.f, f[1] + 4 * i);
         }
-        const int g = (int)((s & 7u) >> 1);
+        // 6-bit (scale, min) pairs 2g and 2g+1 of the block, g = (s % 8) / 2 (langtax/src/quant.rs:8901-8912)
+        const uint32_t g = (s & 7u) >> 1;
+        const uint32_t sh = 16 * (g & 1u);  // pairs 2g, 2g+1 sit in bytes (2g % 4), (2g % 4) + 1 of each header dword
+        const uint32_t a2 = (r.hdr.y >> sh) & 0xffffu, b2 = (r.hdr.z >> sh) & 0xffffu, c2 = (r.hdr.w >> sh) & 0xffffu;
+        const uint32_t up = 0u - (g >> 1);  // all ones for pairs 4..7, which are split over the three dwords
+        auto pick = [&](uint32_t lo, uint32_t hi) { return lo ^ ((lo ^ hi) & up); };
+        const uint32_t s0 = pick(a2 & 63u, (c2 & 15u) | ((a2 >> 2) & 0x30u));
+        const uint32_t s1 = pick((a2 >> 8) & 63u, ((c2 >> 8) & 15u) | ((a2 >> 10) & 0x30u));
+        const uint32_t n0 = pick(b2 & 63u, ((c2 >> 4) & 15u) | ((b2 >> 2) & 0x30u));
+        const uint32_t n1 = pick((b2 >> 8) & 63u, ((c2 >> 12) & 15u) | ((b2 >> 10) & 0x30u));
         const float d = h2f((uint16_t)(r.hdr.x & 0xffffu)), dmin = h2f((uint16_t)(r.hdr.x >> 16));
-        float sc0, m0, sc1, m1;
-        q4k_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * g, sc0, m0);
-        q4k_scale_min(r.hdr.y, r.hdr.z, r.hdr.w, 2 * g + 1, sc1, m1);
+        const float sc0 = (float)s0, sc1 = (float)s1, m0 = (float)n0, m1 = (float)n1;
         scale[0] = d * sc0;
         scale[1] = d * sc1;
         offset[0] = -(dmin * m0);
@@ -1302,13 +1402,28 @@ __device__ __forceinline__ void mm_decode(const MmRaw<T> &raw, uint32_t s, uint4
     }
 }
 
+// LDS of one pipeline stage (one step of 32 columns for the workgroup's 256 rows).
+template <uint32_t T, int TT> struct MmStage {
+    static constexpr bool OFFSET = MmTraits<T>::OFFSET;
+    static constexpr int TOK = 32 * TT;
+    static constexpr int XB_VEC = 12 * TOK;  // [group][part][half][token] x 16 bytes
+    static constexpr size_t CODE = 0;                                   // uint4 [2][2][256]
+    static constexpr size_t SCALE = CODE + (size_t)4 * MM_ROWS * 16;    // float [2][256]
+    static constexpr size_t OFFS = SCALE + (size_t)2 * MM_ROWS * 4;     // float [2][256]
+    static constexpr size_t XB = OFFS + (OFFSET ? (size_t)2 * MM_ROWS * 4 : 0);
+    static constexpr int XB_SLOTS = (XB_VEC + 255) / 256 * 256;        // every thread stores whole vectors, no tail branch
+    static constexpr size_t SX = XB + (size_t)XB_SLOTS * 16;            // float [2][TOK], padded to one per thread
+    static constexpr size_t BYTES = SX + (OFFSET ? (size_t)256 * 4 : 0);
+};
+
 template <uint32_t T, int TT>
-__global__ __launch_bounds__(256) void gemm_mfma_kernel(const MmBatch b) {
-    constexpr bool OFFSET = MmTraits<T>::OFFSET;
-    __shared__ uint4 code_s[2][2][MM_ROWS];   // [group][half of the 16 columns][row]
-    __shared__ float scale_s[2][MM_ROWS];
-    __shared__ float offset_s[OFFSET ? 2 : 1][MM_ROWS];
-    __shared__ float sx_s[OFFSET ? 2 : 1][32 * TT];
+__global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const MmBatch b) {
+    using St = MmStage<T, TT>;
+    constexpr bool OFFSET = St::OFFSET;
+    constexpr bool SAME_SCALE = MmTraits<T>::SAME_SCALE;
+    constexpr int TOK = St::TOK;
+    constexpr int XR = (St::XB_VEC + 255) / 256;  // activation vectors each thread stages per step
+    extern __shared__ __align__(16) uint8_t mm_lds[];
 
     uint32_t j = 0;
     for (uint32_t k = 1; k < b.n_jobs; k++)
@@ -1320,16 +1435,17 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const MmBatch b) {
     local /= job.ksplit;
     const uint32_t tile_t = local % job.tok_tiles, tile_r = local / job.tok_tiles;
 
+    // column shares are cut at multiples of 8 steps (a 256-column super-block)
+    const uint32_t n_units = m.cols / 256;
     const uint32_t n_steps = m.cols / 32;
-    const uint32_t s_begin = (uint32_t)((uint64_t)n_steps * ks / job.ksplit);
-    const uint32_t s_end = (uint32_t)((uint64_t)n_steps * (ks + 1) / job.ksplit);
+    const uint32_t s_begin = n_units ? 8 * (uint32_t)((uint64_t)n_units * ks / job.ksplit) : 0;
+    const uint32_t s_end = n_units && ks + 1 < job.ksplit ? 8 * (uint32_t)((uint64_t)n_units * (ks + 1) / job.ksplit) : n_steps;
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t n = lane & 31u, kh = lane >> 5;
     const uint32_t row0 = tile_r * MM_ROWS;
-    const uint32_t drow = row0 + tid < m.rows ? row0 + tid : m.rows - 1;
-    const uint32_t tok0 = tile_t * 32 * TT;          // first token of the tile within the job
-    const uint32_t slot0 = job.tok_off + tok0;       // same, as a slot of the split activations
+    const uint32_t tok0 = tile_t * TOK;             // first token of the tile within the job
+    const uint32_t slot0 = job.tok_off + tok0;      // same, as a slot of the split activations
     const size_t mpad = b.mpad;
 
     f32x16 acc[2][TT];
@@ -1340,69 +1456,203 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const MmBatch b) {
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[rs][tt][v] = 0.f;
 
-    MmRaw<T> cur;
-    if (s_begin < s_end) mm_load<T>(m, drow, s_begin, cur);
-    for (uint32_t s = s_begin; s < s_end; s++) {
-        {
-            uint4 frag[2][2];
-            float sc[2], of[2];
-            mm_decode<T>(cur, s, frag, sc, of);
+    // Global data of the next DEPTH steps, in registers while earlier steps compute: one
+    // step of one workgroup is only a few KB, far too little to cover HBM latency.  The
+    // 64-token tile has no registers to spare for four slots, and needs them less: its
+    // steps take twice as long.
+    constexpr int DEPTH = TT == 1 ? 4 : 2;
+    // (named variables, not arrays: the ring must stay in registers)
+    MmRaw<T> raw0, raw1, raw2, raw3;
+    struct XbRegs { uint4 v0, v1, v2; };  // XR <= 3 vectors, as named members
+    XbRegs xb0, xb1, xb2, xb3;
+    static_assert(XR <= 3, "XbRegs holds three vectors");
+    float sx0 = 0.f, sx1 = 0.f, sx2 = 0.f, sx3 = 0.f;
+
+    // Offsets are applied once per 32 columns that share them: Q5_1 every step
+    // (one block), Q4_K on even steps (a sub-block spans the same group of two
+    // consecutive steps).
+    auto offset_step = [](uint32_t s) { return T == T_Q5_1 || (s & 1u) == 0; };
+
+    // Every fetch issues the same loads whatever the step and the thread (indices
+    // are clamped instead of branching), so that the number of loads in flight is
+    // known at compile time and a wait for the oldest step does not wait for all.
+    auto fetch = [&](uint32_t s_want, MmRaw<T> &raw, XbRegs &xbr, float &sxr) {
+        const uint32_t s = s_want < s_end ? s_want : s_end - 1;
+        mm_load<T>(m, tile_r, tid, s, raw);
+        const uint4 *src = b.xb + (size_t)s * 12 * mpad + slot0;
 #pragma unroll
-            for (int g = 0; g < 2; g++) {
-                code_s[g][0][tid] = frag[g][0];
-                code_s[g][1][tid] = frag[g][1];
-                scale_s[g][tid] = sc[g];
-                if constexpr (OFFSET) offset_s[g][tid] = of[g];
-            }
-            if constexpr (OFFSET) {
-                if (tid < 2 * 32 * TT) {
-                    const uint32_t g = tid / (32 * TT), i = tid % (32 * TT);
-                    sx_s[g][i] = b.sx[(size_t)(2 * s + g) * mpad + slot0 + i];
-                }
-            }
+        for (int r = 0; r < XR; r++) {
+            uint32_t v = tid + 256 * r;
+            if (XR * 256 != St::XB_VEC) v = v < (uint32_t)St::XB_VEC ? v : (uint32_t)St::XB_VEC - 1;
+            const uint4 val = src[(size_t)(v / TOK) * mpad + v % TOK];
+            if (r == 0) xbr.v0 = val;
+            if (r == 1) xbr.v1 = val;
+            if (r == 2) xbr.v2 = val;
         }
-        if (s + 1 < s_end) mm_load<T>(m, drow, s + 1, cur);
-        __syncthreads();
+        if constexpr (OFFSET) {
+            const uint32_t g = (tid / TOK) & 1u, i = tid % TOK;
+            const uint32_t se = T == T_Q5_1 ? s : s & ~1u;  // Q4_K: the pair of steps of one sub-block
+            const size_t g0 = T == T_Q5_1 ? (size_t)2 * se : (size_t)2 * se + g;
+            const size_t g1 = T == T_Q5_1 ? g0 + 1 : g0 + 2;
+            sxr = b.sx[g0 * mpad + slot0 + i] + b.sx[g1 * mpad + slot0 + i];
+        }
+    };
+    auto store = [&](uint32_t s_want, uint32_t buf, const MmRaw<T> &raw, const XbRegs &xbr, const float &sxr) {
+        const uint32_t s = s_want < s_end ? s_want : s_end - 1;  // past the end: decodes the clamped fetch, never read
+        uint8_t *st = mm_lds + (size_t)buf * St::BYTES;
+        uint4 frag[2][2];
+        float sc[2], of[2];
+        mm_decode<T>(raw, s, frag, sc, of);
+        uint4 *code_s = reinterpret_cast<uint4 *>(st + St::CODE);
+        float *scale_s = reinterpret_cast<float *>(st + St::SCALE);
 #pragma unroll
         for (int g = 0; g < 2; g++) {
-            const size_t gi = (size_t)2 * s + g;
-            bf16x8 wf[2];
-            float sc[2], of[2];
+            code_s[(2 * g) * MM_ROWS + tid] = frag[g][0];
+            code_s[(2 * g + 1) * MM_ROWS + tid] = frag[g][1];
+            scale_s[g * MM_ROWS + tid] = sc[g];
+            if constexpr (OFFSET) reinterpret_cast<float *>(st + St::OFFS)[g * MM_ROWS + tid] = of[g];
+        }
+        uint4 *xb_s = reinterpret_cast<uint4 *>(st + St::XB);
+#pragma unroll
+        for (int r = 0; r < XR; r++) {
+            const uint32_t v = tid + 256 * r;
+            xb_s[v] = r == 0 ? xbr.v0 : r == 1 ? xbr.v1 : xbr.v2;  // slots past XB_VEC are padding
+        }
+        if constexpr (OFFSET) {
+            reinterpret_cast<float *>(st + St::SX)[tid] = sxr;  // read only on offset steps, entries [0, 2 TOK)
+        }
+    };
+    // even_step: s is even (known at compile time: shares of K-quant rows start at a multiple of 8 steps)
+    auto compute = [&](uint32_t s, uint32_t buf, auto even_step) {
+        const uint8_t *st = mm_lds + (size_t)buf * St::BYTES;
+        const uint4 *code_s = reinterpret_cast<const uint4 *>(st + St::CODE);
+        const float *scale_s = reinterpret_cast<const float *>(st + St::SCALE);
+        const float *offs_s = reinterpret_cast<const float *>(st + St::OFFS);
+        const uint4 *xb_s = reinterpret_cast<const uint4 *>(st + St::XB);
+        const float *sx_s = reinterpret_cast<const float *>(st + St::SX);
+        (void)s;
+        constexpr bool with_offset = OFFSET && (T == T_Q5_1 || decltype(even_step)::value);
+        bf16x8 wf[2][2];
+        float sc[2][2], of[2][2];
+#pragma unroll
+        for (int g = 0; g < 2; g++)
 #pragma unroll
             for (int rs = 0; rs < 2; rs++) {
                 const uint32_t r = wave * 64 + rs * 32 + n;
-                wf[rs] = __builtin_bit_cast(bf16x8, code_s[g][kh][r]);
-                sc[rs] = scale_s[g][r];
-                of[rs] = OFFSET ? offset_s[g][r] : 0.f;
+                wf[g][rs] = __builtin_bit_cast(bf16x8, code_s[(2 * g + kh) * MM_ROWS + r]);
+                sc[g][rs] = scale_s[g * MM_ROWS + r];
+                of[g][rs] = OFFSET ? offs_s[g * MM_ROWS + r] : 0.f;
             }
 #pragma unroll
-            for (int tt = 0; tt < TT; tt++) {
-                const uint4 *xp = b.xb + (gi * 6 + kh) * mpad + slot0 + tt * 32 + n;
-                const bf16x8 x_hi = __builtin_bit_cast(bf16x8, xp[0]);
-                const bf16x8 x_mid = __builtin_bit_cast(bf16x8, xp[2 * mpad]);
-                const bf16x8 x_lo = __builtin_bit_cast(bf16x8, xp[4 * mpad]);
-                float sxv[16];
-                if constexpr (OFFSET) {
+        for (int tt = 0; tt < TT; tt++) {
+            // one token tile at a time: interleaving the tiles only lengthens live ranges
+            if (tt > 0) __builtin_amdgcn_sched_barrier(0);
+            bf16x8 xf[2][3];
 #pragma unroll
-                    for (int v = 0; v < 16; v++) sxv[v] = sx_s[g][tt * 32 + 8 * (v >> 2) + 4 * kh + (v & 3)];
+            for (int g = 0; g < 2; g++)
+#pragma unroll
+                for (int p = 0; p < 3; p++)
+                    xf[g][p] = __builtin_bit_cast(bf16x8, xb_s[(g * 6 + 2 * p + kh) * TOK + tt * 32 + n]);
+            // sxv: sums of activations (over the 32 columns an offset covers) of the lane's 16 token rows
+            auto load_sx = [&](int g, float (&sxv)[16]) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float4 t4 = *reinterpret_cast<const float4 *>(sx_s + g * TOK + tt * 32 + 8 * q + 4 * kh);
+                    sxv[4 * q] = t4.x; sxv[4 * q + 1] = t4.y; sxv[4 * q + 2] = t4.z; sxv[4 * q + 3] = t4.w;
                 }
+            };
+            if constexpr (SAME_SCALE) {
+                float sxv[16];
+                if constexpr (with_offset) load_sx(0, sxv);
 #pragma unroll
                 for (int rs = 0; rs < 2; rs++) {
                     f32x16 p;
 #pragma unroll
                     for (int v = 0; v < 16; v++) p[v] = 0.f;
-                    p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_lo, wf[rs], p, 0, 0, 0);
-                    p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_mid, wf[rs], p, 0, 0, 0);
-                    p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x_hi, wf[rs], p, 0, 0, 0);
 #pragma unroll
-                    for (int v = 0; v < 16; v++) {
-                        acc[rs][tt][v] = fmaf(sc[rs], p[v], acc[rs][tt][v]);
-                        if constexpr (OFFSET) acc[rs][tt][v] = fmaf(of[rs], sxv[v], acc[rs][tt][v]);
+                    for (int g = 0; g < 2; g++) {
+                        p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[g][2], wf[g][rs], p, 0, 0, 0);
+                        p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[g][1], wf[g][rs], p, 0, 0, 0);
+                        p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[g][0], wf[g][rs], p, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int v = 0; v < 16; v++) acc[rs][tt][v] = fmaf(sc[0][rs], p[v], acc[rs][tt][v]);
+                    if constexpr (with_offset) {
+#pragma unroll
+                        for (int v = 0; v < 16; v++) acc[rs][tt][v] = fmaf(of[0][rs], sxv[v], acc[rs][tt][v]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int g = 0; g < 2; g++) {
+                    float sxv[16];
+                    if constexpr (with_offset) load_sx(g, sxv);
+#pragma unroll
+                    for (int rs = 0; rs < 2; rs++) {
+                        f32x16 p;
+#pragma unroll
+                        for (int v = 0; v < 16; v++) p[v] = 0.f;
+                        p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[g][2], wf[g][rs], p, 0, 0, 0);
+                        p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[g][1], wf[g][rs], p, 0, 0, 0);
+                        p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[g][0], wf[g][rs], p, 0, 0, 0);
+#pragma unroll
+                        for (int v = 0; v < 16; v++) acc[rs][tt][v] = fmaf(sc[g][rs], p[v], acc[rs][tt][v]);
+                        if constexpr (with_offset) {
+#pragma unroll
+                            for (int v = 0; v < 16; v++) acc[rs][tt][v] = fmaf(of[g][rs], sxv[v], acc[rs][tt][v]);
+                        }
                     }
                 }
             }
         }
-        __syncthreads();
+    };
+
+    if (s_begin < s_end) {
+        // No branch inside a step: the compiler then knows how many loads are in flight
+        // and waits only for the oldest ring slot.  Step s computes from LDS stage
+        // (s - s_begin) & 1 while step s + 1 is decoded into the other stage from its
+        // ring slot, which is then refilled for step s + 1 + DEPTH.
+#define NH_MM_STEP(d, RAW, XB, SX)                                                     \
+    {                                                                                  \
+        store(base + d + 1, (d + 1) & 1, RAW, XB, SX);                                 \
+        fetch(base + d + 1 + DEPTH, RAW, XB, SX);                                      \
+        __builtin_amdgcn_sched_barrier(0);                                             \
+        compute(base + d, d & 1, std::integral_constant<bool, ((d) & 1) == 0>{});      \
+        __builtin_amdgcn_sched_barrier(0);                                             \
+        __syncthreads();                                                               \
+    }
+        uint32_t base = s_begin;
+        if constexpr (DEPTH == 4) {
+            fetch(s_begin, raw0, xb0, sx0);
+            fetch(s_begin + 1, raw1, xb1, sx1);
+            fetch(s_begin + 2, raw2, xb2, sx2);
+            fetch(s_begin + 3, raw3, xb3, sx3);
+            store(s_begin, 0, raw0, xb0, sx0);
+            fetch(s_begin + 4, raw0, xb0, sx0);
+            __syncthreads();
+            for (; base + 4 <= s_end; base += 4) {
+                NH_MM_STEP(0, raw1, xb1, sx1)
+                NH_MM_STEP(1, raw2, xb2, sx2)
+                NH_MM_STEP(2, raw3, xb3, sx3)
+                NH_MM_STEP(3, raw0, xb0, sx0)
+            }
+            // at most three steps left (column counts that are not a multiple of 128)
+            if (base < s_end) NH_MM_STEP(0, raw1, xb1, sx1)
+            if (base + 1 < s_end) NH_MM_STEP(1, raw2, xb2, sx2)
+            if (base + 2 < s_end) NH_MM_STEP(2, raw3, xb3, sx3)
+        } else {
+            fetch(s_begin, raw0, xb0, sx0);
+            fetch(s_begin + 1, raw1, xb1, sx1);
+            store(s_begin, 0, raw0, xb0, sx0);
+            fetch(s_begin + 2, raw0, xb0, sx0);
+            __syncthreads();
+            for (; base + 2 <= s_end; base += 2) {
+                NH_MM_STEP(0, raw1, xb1, sx1)
+                NH_MM_STEP(1, raw0, xb0, sx0)
+            }
+            if (base < s_end) NH_MM_STEP(0, raw1, xb1, sx1)
+        }
+#undef NH_MM_STEP
     }
 
     // D[i][j]: lane holds weight row j = lane % 32 and token rows i = 8 (v / 4) + 4 (lane / 32) + v % 4.
@@ -1424,12 +1674,27 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const MmBatch b) {
 // y = sum over the column shares, in share order.
 __global__ __launch_bounds__(256) void mm_reduce_kernel(const MmBatch b) {
     const MmJob &job = b.job[blockIdx.y];
-    const size_t total = (size_t)job.tokens * job.m.rows;
     if (job.ksplit < 2) return;
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
-        float s = job.part[i];
-        for (uint32_t k = 1; k < job.ksplit; k++) s += job.part[(size_t)k * total + i];
-        job.y[i] = s;
+    const size_t total = (size_t)job.tokens * job.m.rows;
+    const size_t first = (size_t)blockIdx.x * 256 + threadIdx.x, stride = (size_t)gridDim.x * 256;
+    if ((total & 3) == 0 && (reinterpret_cast<uintptr_t>(job.y) & 15) == 0) {
+        const float4 *part = reinterpret_cast<const float4 *>(job.part);
+        float4 *y = reinterpret_cast<float4 *>(job.y);
+        const size_t total4 = total / 4;
+        for (size_t i = first; i < total4; i += stride) {
+            float4 s = part[i];
+            for (uint32_t k = 1; k < job.ksplit; k++) {
+                const float4 t = part[(size_t)k * total4 + i];
+                s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+            }
+            y[i] = s;
+        }
+    } else {
+        for (size_t i = first; i < total; i += stride) {
+            float s = job.part[i];
+            for (uint32_t k = 1; k < job.ksplit; k++) s += job.part[(size_t)k * total + i];
+            job.y[i] = s;
+        }
     }
 }
 
@@ -1689,9 +1954,9 @@ static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *co
         // The column split of a product depends on that product alone, so that its
         // result does not change with what else shares the launch.
         const uint32_t tiles = job.tok_tiles * ((mats[j].rows + MM_ROWS - 1) / MM_ROWS);
-        uint32_t ks = (uint32_t)g_cu_count / tiles;
-        if (ks > n_steps / 4) ks = n_steps / 4;
-        if (ks > 16) ks = 16;
+        uint32_t ks = (uint32_t)(2 * g_cu_count) / tiles;  // two workgroups per CU
+        if (ks > n_steps / 8) ks = n_steps / 8;            // shares are whole 256-column units
+        if (ks > 32) ks = 32;
         if (ks < 1) ks = 1;
         job.ksplit = ks;
         job.pad = 0;
@@ -1713,6 +1978,20 @@ static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *co
     p.part_bytes = part;
 }
 
+template <uint32_t T, int TT> static hipError_t launch_mm_main(hipStream_t stream, const MmBatch &b) {
+    constexpr size_t lds = 2 * MmStage<T, TT>::BYTES;  // two pipeline stages
+    auto kern = gemm_mfma_kernel<T, TT>;
+    static bool configured = false;
+    if (lds > 48 * 1024 && !configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)lds);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(b.total_wgs), dim3(256), lds, stream, b);
+    return hipGetLastError();
+}
+
 template <uint32_t T>
 static hipError_t launch_mm_t(hipStream_t stream, MmPlan &p, void *ws, size_t ws_bytes) {
     if (p.xb_bytes + p.sx_bytes + p.part_bytes > ws_bytes) return hipErrorInvalidValue;
@@ -1729,11 +2008,9 @@ static hipError_t launch_mm_t(hipStream_t stream, MmPlan &p, void *ws, size_t ws
     const size_t split_threads = (size_t)p.n_groups * b.mpad;
     hipLaunchKernelGGL(mm_xsplit_kernel<T>, dim3((unsigned)((split_threads + 255) / 256)), dim3(256), 0, stream, b,
                        p.n_groups);
-    if (p.tt == 1)
-        hipLaunchKernelGGL((gemm_mfma_kernel<T, 1>), dim3(b.total_wgs), dim3(256), 0, stream, b);
-    else
-        hipLaunchKernelGGL((gemm_mfma_kernel<T, 2>), dim3(b.total_wgs), dim3(256), 0, stream, b);
-    if (b.any_split) hipLaunchKernelGGL(mm_reduce_kernel, dim3(64, b.n_jobs), dim3(256), 0, stream, b);
+    hipError_t e = p.tt == 1 ? launch_mm_main<T, 1>(stream, b) : launch_mm_main<T, 2>(stream, b);
+    if (e != hipSuccess) return e;
+    if (b.any_split) hipLaunchKernelGGL(mm_reduce_kernel, dim3(512, b.n_jobs), dim3(256), 0, stream, b);
     return hipGetLastError();
 }
 
@@ -1798,8 +2075,8 @@ size_t gemm_workspace_bytes(const MatView *mats, const uint32_t *tokens, uint32_
     return need;
 }
 
-hipError_t launch_gemm_groups(hipStream_t stream, const MatView *mats, const uint32_t *tokens, const float *const *xs,
-                              float *const *ys, uint32_t n, void *ws, size_t ws_bytes) {
+hipError_t launch_gemm_groups(hipStream_t stream, const MatView *mats, const MatView *tiled, const uint32_t *tokens,
+                              const float *const *xs, float *const *ys, uint32_t n, void *ws, size_t ws_bytes) {
     for (uint32_t g = 0; g < n;) {
         if (tokens[g] == 0 || mats[g].rows == 0) { g++; continue; }
         const uint32_t run = mm_run(mats, tokens, n, g);
@@ -1809,7 +2086,7 @@ hipError_t launch_gemm_groups(hipStream_t stream, const MatView *mats, const uin
             g++;
         } else {
             MmPlan p;
-            mm_plan(mats + g, tokens + g, xs + g, ys + g, run, p);
+            mm_plan(tiled + g, tokens + g, xs + g, ys + g, run, p);
             e = launch_mm(stream, p, ws, ws_bytes);
             g += run;
         }
@@ -1847,9 +2124,9 @@ hipError_t launch_gemv_multi(hipStream_t stream, const MatView *mats, float *con
     }
 }
 
-hipError_t launch_gemm(hipStream_t stream, const MatView &m, uint32_t tokens, const float *x, float *y, void *ws,
-                       size_t ws_bytes) {
-    return launch_gemm_groups(stream, &m, &tokens, &x, &y, 1, ws, ws_bytes);
+hipError_t launch_gemm(hipStream_t stream, const MatView &m, const MatView &tiled, uint32_t tokens, const float *x,
+                       float *y, void *ws, size_t ws_bytes) {
+    return launch_gemm_groups(stream, &m, &tiled, &tokens, &x, &y, 1, ws, ws_bytes);
 }
 
 }  // namespace nh

@@ -115,4 +115,50 @@ inline PlaneSpec plane_spec(uint32_t t, size_t rows, size_t cols) {
     return s;
 }
 
+// Second copy of a quantized matrix for products of two or more tokens, where one
+// thread decodes one row: rows are interleaved in tiles of 256 so that the 256
+// threads of a workgroup, each fetching the same field of its own row, read
+// one contiguous run.  Plane k holds units of unit[k] bytes, per_row[k] of them per
+// row, unit i of row r at
+//     ((r / 256 * per_row[k] + i) * 256 + r % 256) * unit[k].
+//
+//   Q8_0 : codes 16 B x 2 nb | d 2 B x nb
+//   Q4_0 : codes 16 B x nb   | d 2 B x nb
+//   Q5_0 : codes 16 B x nb   | qh 4 B x nb | d 2 B x nb
+//   Q5_1 : codes 16 B x nb   | qh 4 B x nb | (d, m) 4 B x nb
+//   Q4_K : codes 16 B x 8 nb | header 16 B x nb
+//   Q6_K : ql 16 B x 8 nb    | qh 16 B x 4 nb | sc 8 B x 2 nb | d 2 B x nb
+// (code units in the order of the GGUF block).  F32/F16 have no such copy.
+constexpr uint32_t TILE_ROWS = 256;
+
+struct TiledSpec {
+    size_t unit[4], per_row[4];
+    size_t offset[4];
+    size_t total;  // 0: this dtype has no tiled copy
+};
+
+inline TiledSpec tiled_spec(uint32_t t, size_t rows, size_t cols) {
+    TiledSpec s = {};
+    if (t == T_F32 || t == T_F16 || !type_supported(t)) return s;
+    const size_t nb = cols / block_elems(t);
+    auto set = [&](int k, size_t unit, size_t per_row) { s.unit[k] = unit; s.per_row[k] = per_row; };
+    switch (t) {
+    case T_Q8_0: set(0, 16, 2 * nb); set(1, 2, nb); break;
+    case T_Q4_0: set(0, 16, nb); set(1, 2, nb); break;
+    case T_Q5_0: set(0, 16, nb); set(1, 4, nb); set(2, 2, nb); break;
+    case T_Q5_1: set(0, 16, nb); set(1, 4, nb); set(2, 4, nb); break;
+    case T_Q4_K: set(0, 16, 8 * nb); set(1, 16, nb); break;
+    case T_Q6_K: set(0, 16, 8 * nb); set(1, 16, 4 * nb); set(2, 8, 2 * nb); set(3, 2, nb); break;
+    default: break;
+    }
+    const size_t tiles = (rows + TILE_ROWS - 1) / TILE_ROWS;
+    size_t off = 0;
+    for (int k = 0; k < 4; k++) {
+        s.offset[k] = off;
+        off = round_up(off + tiles * s.per_row[k] * TILE_ROWS * s.unit[k], 256);
+    }
+    s.total = off;
+    return s;
+}
+
 }  // namespace nh

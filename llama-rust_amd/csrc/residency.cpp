@@ -166,8 +166,8 @@ int resident(State &s, uint32_t type, size_t rows, size_t cols, const uint8_t *w
         }
     }
     s.misses++;
-    nh::PlaneSpec ps = nh::plane_spec(type, rows, cols);
-    size_t bytes = ps.total + w_len;
+    // both device copies of the matrix (matview.h) plus the host copy kept for the identity check
+    size_t bytes = nh::plane_spec(type, rows, cols).total + nh::tiled_spec(type, rows, cols).total + w_len;
     if (bytes < w_len) return qfail(LNH_ERR_INVALID, "resident matrix size overflow");
     while (!s.cache.empty() && admission_requires_eviction(s.bytes, bytes, s.limit)) {
         s.bytes = s.bytes > s.cache.front().bytes ? s.bytes - s.cache.front().bytes : 0;
