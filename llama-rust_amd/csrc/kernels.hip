@@ -78,14 +78,19 @@ __global__ void repack_blocks(MutView v, const uint8_t *__restrict__ src, size_t
     size_t total = (size_t)v.rows * v.nb;
     if (idx >= total) return;
     size_t r = idx / v.nb, b = idx % v.nb;
+    // code pieces of the 32-column dtypes: piece-major when the row is whole units (matview.h)
+    const bool major = piece_major(v.type, v.cols);
+    const size_t units = v.cols / unit_cols(v.type);
     switch (v.type) {
     case T_Q8_0: {
         const uint8_t *s = src + r * src_row_bytes + b * 34;
         uint8_t *d = v.p1 + r * v.s1 + b * 2;
         d[0] = s[0];
         d[1] = s[1];
-        uint8_t *q = v.p0 + r * v.s0 + b * 32;
-        for (int i = 0; i < 32; i++) q[i] = s[2 + i];
+        for (int h = 0; h < 2; h++) {
+            uint8_t *q = v.p0 + r * v.s0 + piece_offset(major, units, 2 * b + h);
+            for (int i = 0; i < 16; i++) q[i] = s[2 + 16 * h + i];
+        }
         break;
     }
     case T_Q4_0: {
@@ -93,7 +98,7 @@ __global__ void repack_blocks(MutView v, const uint8_t *__restrict__ src, size_t
         uint8_t *d = v.p1 + r * v.s1 + b * 2;
         d[0] = s[0];
         d[1] = s[1];
-        uint8_t *q = v.p0 + r * v.s0 + b * 16;
+        uint8_t *q = v.p0 + r * v.s0 + piece_offset(major, units, b);
         for (int i = 0; i < 16; i++) q[i] = s[2 + i];
         break;
     }
@@ -104,7 +109,7 @@ __global__ void repack_blocks(MutView v, const uint8_t *__restrict__ src, size_t
         d[1] = s[1];
         uint8_t *h = v.p1 + r * v.s1 + b * 4;
         for (int i = 0; i < 4; i++) h[i] = s[2 + i];
-        uint8_t *q = v.p0 + r * v.s0 + b * 16;
+        uint8_t *q = v.p0 + r * v.s0 + piece_offset(major, units, b);
         for (int i = 0; i < 16; i++) q[i] = s[6 + i];
         break;
     }
@@ -114,7 +119,7 @@ __global__ void repack_blocks(MutView v, const uint8_t *__restrict__ src, size_t
         for (int i = 0; i < 4; i++) d[i] = s[i];
         uint8_t *h = v.p1 + r * v.s1 + b * 4;
         for (int i = 0; i < 4; i++) h[i] = s[4 + i];
-        uint8_t *q = v.p0 + r * v.s0 + b * 16;
+        uint8_t *q = v.p0 + r * v.s0 + piece_offset(major, units, b);
         for (int i = 0; i < 16; i++) q[i] = s[8 + i];
         break;
     }
@@ -342,17 +347,17 @@ template <uint32_t T> __device__ __forceinline__ void load_raw(const MatView &m,
     if constexpr (T == T_F32 || T == T_F16) {
         r.q = *reinterpret_cast<const uint4 *>(m.p0 + ro * m.s0 + (size_t)c * 16);
     } else if constexpr (T == T_Q8_0) {
-        r.q = *reinterpret_cast<const uint4 *>(m.p0 + ro * m.s0 + (size_t)c * 16);
+        r.q = *reinterpret_cast<const uint4 *>(m.p0 + ro * m.s0 + piece_offset(piece_major(T, m.cols), m.cols / unit_cols(T), c));
         r.d = *reinterpret_cast<const uint16_t *>(m.p1 + ro * m.s1 + (size_t)(c >> 1) * 2);
     } else if constexpr (T == T_Q4_0) {
-        r.q = *reinterpret_cast<const uint4 *>(m.p0 + ro * m.s0 + (size_t)c * 16);
+        r.q = *reinterpret_cast<const uint4 *>(m.p0 + ro * m.s0 + piece_offset(piece_major(T, m.cols), m.cols / unit_cols(T), c));
         r.d = *reinterpret_cast<const uint16_t *>(m.p1 + ro * m.s1 + (size_t)c * 2);
     } else if constexpr (T == T_Q5_0) {
-        r.q = *reinterpret_cast<const uint4 *>(m.p0 + ro * m.s0 + (size_t)c * 16);
+        r.q = *reinterpret_cast<const uint4 *>(m.p0 + ro * m.s0 + piece_offset(piece_major(T, m.cols), m.cols / unit_cols(T), c));
         r.qh = *reinterpret_cast<const uint32_t *>(m.p1 + ro * m.s1 + (size_t)c * 4);
         r.d = *reinterpret_cast<const uint16_t *>(m.p2 + ro * m.s2 + (size_t)c * 2);
     } else if constexpr (T == T_Q5_1) {
-        r.q = *reinterpret_cast<const uint4 *>(m.p0 + ro * m.s0 + (size_t)c * 16);
+        r.q = *reinterpret_cast<const uint4 *>(m.p0 + ro * m.s0 + piece_offset(piece_major(T, m.cols), m.cols / unit_cols(T), c));
         r.qh = *reinterpret_cast<const uint32_t *>(m.p1 + ro * m.s1 + (size_t)c * 4);
         r.dm = *reinterpret_cast<const uint32_t *>(m.p2 + ro * m.s2 + (size_t)c * 4);
     } else if constexpr (T == T_Q4_K) {
@@ -1009,6 +1014,225 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q6k_kernel(const GemvBatch b)
     }
 }
 
+// ------------------------------------------------------------------ Q8_0 / Q4_0 / Q5_0 / Q5_1 GEMV: one lane per unit
+//
+// Same structure as the Q4_K kernel, for the dtypes with 32-column blocks.  A lane
+// owns one unit of one row: 8 consecutive blocks (256 columns) of Q4_0/Q5_0/Q5_1 or
+// 4 blocks (128 columns) of Q8_0, i.e. 8 code pieces of 16 bytes (piece-major, see
+// matview.h) plus the unit's scales, which are contiguous in their plane.  x sits in
+// LDS in column order, one float4 row per 4 columns of a unit, padded like the
+// Q4_K kernel's.  Code biases (8, 16, 128) and Q5_1's offsets go through the
+// per-block sums of x:  sum_k d (q_k - bias) x_k = d (sum_k q_k x_k - bias sum_k x_k)
+// (langtax/src/quant.rs:7511-7541, 7734-7765, 7884-7950, 8046-8130).
+
+template <uint32_t T> struct B32Geo {
+    static constexpr int UC = T == T_Q8_0 ? 128 : 256;  // columns per unit
+    static constexpr int NBLK = UC / 32;                // blocks per unit
+    static constexpr int XV = UC / 32;                  // float4 of x per code piece
+};
+template <uint32_t T> struct B32Unit;
+template <> struct B32Unit<T_Q8_0> { uint4 q[8]; uint2 d; };
+template <> struct B32Unit<T_Q4_0> { uint4 q[8]; uint4 d; };
+template <> struct B32Unit<T_Q5_0> { uint4 q[8]; uint4 qh[2]; uint4 d; };
+template <> struct B32Unit<T_Q5_1> { uint4 q[8]; uint4 qh[2]; uint4 dm[2]; };
+
+template <uint32_t T, int LB, int NW, bool FP8>
+__global__ __launch_bounds__(NW * 64, (T == T_Q5_0 || T == T_Q5_1) ? 3 : 4) void gemv_b32_kernel(const GemvBatch b, const float nib_mul, const float nib_unit) {
+    using G = B32Geo<T>;
+    constexpr uint32_t RS = 64 / LB;           // rows per wavefront step = rows per row group
+    constexpr uint32_t XROW = LB * 4 + 4;      // floats per LDS row: LB float4 plus one of padding
+    constexpr uint32_t XS_FLOATS = (G::UC / 4) * XROW;
+    extern __shared__ __align__(16) float lds[];
+    const uint32_t cols = b.job[0].m.cols;
+    const uint32_t nu = cols / G::UC;                 // units per row
+    const uint32_t n_iter = (nu + LB - 1) / LB;
+    float *xs = lds;                                   // [it][column / 4 of the unit][unit % LB] float4
+    float *ssum = lds + (size_t)n_iter * XS_FLOATS;    // [it][block of the unit][unit % LB]: sum of x over the block
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t total_waves = gridDim.x * NW;
+    const uint32_t sub_row = lane / LB, b0 = lane % LB;
+    // A wavefront takes whole row groups (every total_waves-th one) and walks the
+    // n_iter unit columns of each in turn, so that a row's sum stays in one lane.
+    struct Pos {
+        uint32_t g, it;
+    };
+    auto advance = [&](Pos p) {
+        p.it++;
+        if (p.it == n_iter) {
+            p.it = 0;
+            p.g += total_waves;
+        }
+        return p;
+    };
+    auto valid = [&](const Pos &p) { return p.g < b.total_rgs; };
+
+    struct Where {
+        const MatView *m;
+        float *y;
+        uint32_t row0;
+    };
+    auto locate = [&](uint32_t g) {
+        uint32_t j = 0;
+        while (j + 1 < b.n_jobs && g >= b.job[j + 1].rg_begin) j++;
+        Where w;
+        w.m = &b.job[j].m;
+        w.y = b.job[j].y;
+        w.row0 = (g - b.job[j].rg_begin) * RS;
+        return w;
+    };
+    auto fetch = [&](const Pos &p, B32Unit<T> &o) {
+        const uint32_t it = p.it;
+        const Where w = locate(p.g < b.total_rgs ? p.g : b.total_rgs - 1);
+        const MatView &m = *w.m;
+        uint32_t row = w.row0 + sub_row;
+        row = row < m.rows ? row : m.rows - 1;
+        uint32_t un = it * LB + b0;
+        un = un < nu ? un : nu - 1;
+        const uint8_t *q = m.p0 + (size_t)row * m.s0 + (size_t)un * 16;
+#pragma unroll
+        for (int cc = 0; cc < 8; cc++) o.q[cc] = *reinterpret_cast<const uint4 *>(q + (size_t)cc * nu * 16);
+        if constexpr (T == T_Q8_0) {
+            o.d = *reinterpret_cast<const uint2 *>(m.p1 + (size_t)row * m.s1 + (size_t)un * 8);
+        } else if constexpr (T == T_Q4_0) {
+            o.d = *reinterpret_cast<const uint4 *>(m.p1 + (size_t)row * m.s1 + (size_t)un * 16);
+        } else {
+            const uint4 *h = reinterpret_cast<const uint4 *>(m.p1 + (size_t)row * m.s1 + (size_t)un * 32);
+            o.qh[0] = h[0];
+            o.qh[1] = h[1];
+            if constexpr (T == T_Q5_0) {
+                o.d = *reinterpret_cast<const uint4 *>(m.p2 + (size_t)row * m.s2 + (size_t)un * 16);
+            } else {
+                const uint4 *dm = reinterpret_cast<const uint4 *>(m.p2 + (size_t)row * m.s2 + (size_t)un * 32);
+                o.dm[0] = dm[0];
+                o.dm[1] = dm[1];
+            }
+        }
+    };
+
+    Pos pa = {blockIdx.x * NW + wave, 0};
+    B32Unit<T> ua, ub;
+    // Stage x once per workgroup; eight consecutive lanes hold one 32-column block.
+    auto stage = [&](uint32_t col, const float4 v) {
+        const uint32_t un = col / G::UC, e = col % G::UC, it = un / LB, bl = un % LB;
+        *reinterpret_cast<float4 *>(xs + (size_t)it * XS_FLOATS + (e >> 2) * XROW + bl * 4) = v;
+        float sm = (v.x + v.y) + (v.z + v.w);
+#define NH_DPP_ADD(ctrl) sm += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), ctrl, 0xf, 0xf, false))
+        NH_DPP_ADD(0xb1);
+        NH_DPP_ADD(0x4e);
+        NH_DPP_ADD(0x141);
+#undef NH_DPP_ADD
+        if ((lane & 7u) == 0) ssum[(it * G::NBLK + (e >> 5)) * LB + bl] = sm;
+    };
+    constexpr int NXV = (LB * G::UC / 4 + NW * 64 - 1) / (NW * 64);  // float4 per thread for LB units of x
+    if (n_iter == 1) {
+        float4 xv[NXV];
+#pragma unroll
+        for (int k = 0; k < NXV; k++) {
+            const uint32_t col = (tid + k * NW * 64) * 4;
+            xv[k] = *reinterpret_cast<const float4 *>(b.x + (col < cols ? col : 0));  // branch-free: stays first
+        }
+        __builtin_amdgcn_sched_barrier(0);  // keep the x loads ahead of the weight loads in the queue
+        fetch(pa, ua);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < NXV; k++) {
+            const uint32_t col = (tid + k * NW * 64) * 4;
+            if (col < LB * G::UC) stage(col, col < cols ? xv[k] : make_float4(0.f, 0.f, 0.f, 0.f));
+        }
+        __syncthreads();
+    } else {
+        for (uint32_t col = tid * 4; col < n_iter * LB * G::UC; col += NW * 64 * 4)
+            stage(col, col < cols ? *reinterpret_cast<const float4 *>(b.x + col) : make_float4(0.f, 0.f, 0.f, 0.f));
+        __syncthreads();
+        if (valid(pa)) fetch(pa, ua);
+    }
+
+    float acc = 0.f;
+    auto consume = [&](const Pos &p, const B32Unit<T> &q) {
+        const uint32_t g = p.g, it = p.it;
+        const bool active = it * LB + b0 < nu;
+        const float *xb = xs + (size_t)it * XS_FLOATS + b0 * 4;
+        const float *sp = ssum + (size_t)it * G::NBLK * LB + b0;
+        float t[G::NBLK];
+#pragma unroll
+        for (int k = 0; k < G::NBLK; k++) t[k] = 0.f;
+        uint32_t qh[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if constexpr (T == T_Q5_0 || T == T_Q5_1) {
+            qh[0] = q.qh[0].x; qh[1] = q.qh[0].y; qh[2] = q.qh[0].z; qh[3] = q.qh[0].w;
+            qh[4] = q.qh[1].x; qh[5] = q.qh[1].y; qh[6] = q.qh[1].z; qh[7] = q.qh[1].w;
+        }
+#pragma unroll
+        for (int cc = 0; cc < 8; cc++) {
+            float x[4 * G::XV];
+#pragma unroll
+            for (int i = 0; i < G::XV; i++) {
+                float4 v = *reinterpret_cast<const float4 *>(xb + (cc * G::XV + i) * XROW);
+                x[4 * i] = v.x; x[4 * i + 1] = v.y; x[4 * i + 2] = v.z; x[4 * i + 3] = v.w;
+            }
+            const uint32_t w[4] = {q.q[cc].x, q.q[cc].y, q.q[cc].z, q.q[cc].w};
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                if constexpr (T == T_Q8_0) {
+                    // signed byte + 128 as an unsigned byte; the 128 comes back out through the sum of x
+                    t[cc >> 1] = dot4_ub(w[d] ^ 0x80808080u, x + 4 * d, t[cc >> 1]);
+                } else if constexpr (T == T_Q4_0) {
+                    t[cc] = dot4_nib<FP8>(w[d] & 0x0f0f0f0fu, x + 4 * d, t[cc]);
+                    t[cc] = dot4_nib<FP8>((w[d] >> 4) & 0x0f0f0f0fu, x + 16 + 4 * d, t[cc]);
+                } else {
+                    t[cc] = dot4_ub(q5_bytes(w[d] & 0x0f0f0f0fu, qh[cc], 4 * d), x + 4 * d, t[cc]);
+                    t[cc] = dot4_ub(q5_bytes((w[d] >> 4) & 0x0f0f0f0fu, qh[cc], 16 + 4 * d), x + 16 + 4 * d, t[cc]);
+                }
+            }
+        }
+        float part = 0.f;
+        if constexpr (T == T_Q8_0) {
+            const uint32_t dd[2] = {q.d.x, q.d.y};
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const float d = h2f((uint16_t)(dd[k >> 1] >> (16 * (k & 1))));
+                part = fmaf(d, fmaf(-128.f, sp[k * LB], t[k]), part);
+            }
+        } else if constexpr (T == T_Q4_0 || T == T_Q5_0) {
+            const uint32_t dd[4] = {q.d.x, q.d.y, q.d.z, q.d.w};
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const float d = h2f((uint16_t)(dd[k >> 1] >> (16 * (k & 1))));
+                if constexpr (T == T_Q4_0)  // t holds nib_unit * sum n x when the fp8 unpack is in use
+                    part = fmaf(d * nib_mul, fmaf(-8.f * nib_unit, sp[k * LB], t[k]), part);
+                else
+                    part = fmaf(d, fmaf(-16.f, sp[k * LB], t[k]), part);
+            }
+        } else {
+            const uint32_t dm[8] = {q.dm[0].x, q.dm[0].y, q.dm[0].z, q.dm[0].w, q.dm[1].x, q.dm[1].y, q.dm[1].z, q.dm[1].w};
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                part = fmaf(h2f((uint16_t)(dm[k] & 0xffffu)), t[k], part);
+                part = fmaf(h2f((uint16_t)(dm[k] >> 16)), sp[k * LB], part);
+            }
+        }
+        acc += active ? part : 0.f;
+        if (it + 1 == n_iter) {  // row group complete
+            const Where w = locate(g);
+            const float tot = group_sum_dpp<LB>(acc);
+            const uint32_t row = w.row0 + sub_row;
+            if (b0 == LB - 1 && row < w.m->rows) w.y[row] = tot;
+            acc = 0.f;
+        }
+    };
+
+    while (valid(pa)) {
+        const Pos pb = advance(pa);
+        if (valid(pb)) fetch(pb, ub);
+        consume(pa, ua);
+        if (!valid(pb)) break;
+        pa = advance(pb);
+        if (valid(pa)) fetch(pa, ua);
+        consume(pb, ub);
+    }
+}
+
 // ------------------------------------------------------------------ tiled GEMM (any token count)
 //
 // Eight consecutive decoded weights of one row starting at column k0 (k0 % 8 == 0).
@@ -1028,7 +1252,8 @@ template <uint32_t T> __device__ __forceinline__ void dequant8(const MatView &m,
         }
     } else if constexpr (T == T_Q8_0) {
         uint32_t b = k0 >> 5, j = k0 & 31;
-        uint2 q = *reinterpret_cast<const uint2 *>(m.p0 + ro * m.s0 + (size_t)b * 32 + j);
+        uint2 q = *reinterpret_cast<const uint2 *>(m.p0 + ro * m.s0 +
+                                                   piece_offset(piece_major(T, m.cols), m.cols / unit_cols(T), 2 * b + (j >> 4)) + (j & 15));
         float d = h2f(*reinterpret_cast<const uint16_t *>(m.p1 + ro * m.s1 + (size_t)b * 2));
 #pragma unroll
         for (int k = 0; k < 4; k++) {
@@ -1038,7 +1263,8 @@ template <uint32_t T> __device__ __forceinline__ void dequant8(const MatView &m,
     } else if constexpr (T == T_Q4_0 || T == T_Q5_0 || T == T_Q5_1) {
         // element e = j + i of block b: nibble of byte (e & 15), high nibble when e >= 16
         uint32_t b = k0 >> 5, j = k0 & 31, byte0 = j & 15;
-        uint2 q = *reinterpret_cast<const uint2 *>(m.p0 + ro * m.s0 + (size_t)b * 16 + byte0);
+        uint2 q = *reinterpret_cast<const uint2 *>(m.p0 + ro * m.s0 +
+                                                   piece_offset(piece_major(T, m.cols), m.cols / unit_cols(T), b) + byte0);
         uint32_t sh = j >= 16 ? 4u : 0u;
         uint32_t n0 = (q.x >> sh) & 0x0f0f0f0fu, n1 = (q.y >> sh) & 0x0f0f0f0fu;
         if constexpr (T == T_Q4_0) {
@@ -1671,31 +1897,39 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const MmBatch b) {
     }
 }
 
-// y = sum over the column shares, in share order.
+// y = sum over the column shares, in share order.  The loads of one element's
+// shares are independent and issued eight at a time; the additions keep the order.
+template <typename V> __device__ __forceinline__ V mm_add(V a, V b);
+template <> __device__ __forceinline__ float mm_add<float>(float a, float b) { return a + b; }
+template <> __device__ __forceinline__ float4 mm_add<float4>(float4 a, float4 b) {
+    return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
+}
+template <typename V>
+__device__ __forceinline__ void mm_reduce_span(const V *part, V *y, size_t total, uint32_t ksplit, size_t first, size_t stride) {
+    for (size_t i = first; i < total; i += stride) {
+        V s = part[i];
+        uint32_t k = 1;
+        for (; k + 8 <= ksplit; k += 8) {
+            V t[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) t[u] = part[(size_t)(k + u) * total + i];
+#pragma unroll
+            for (int u = 0; u < 8; u++) s = mm_add(s, t[u]);
+        }
+        for (; k < ksplit; k++) s = mm_add(s, part[(size_t)k * total + i]);
+        y[i] = s;
+    }
+}
 __global__ __launch_bounds__(256) void mm_reduce_kernel(const MmBatch b) {
     const MmJob &job = b.job[blockIdx.y];
     if (job.ksplit < 2) return;
     const size_t total = (size_t)job.tokens * job.m.rows;
     const size_t first = (size_t)blockIdx.x * 256 + threadIdx.x, stride = (size_t)gridDim.x * 256;
-    if ((total & 3) == 0 && (reinterpret_cast<uintptr_t>(job.y) & 15) == 0) {
-        const float4 *part = reinterpret_cast<const float4 *>(job.part);
-        float4 *y = reinterpret_cast<float4 *>(job.y);
-        const size_t total4 = total / 4;
-        for (size_t i = first; i < total4; i += stride) {
-            float4 s = part[i];
-            for (uint32_t k = 1; k < job.ksplit; k++) {
-                const float4 t = part[(size_t)k * total4 + i];
-                s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
-            }
-            y[i] = s;
-        }
-    } else {
-        for (size_t i = first; i < total; i += stride) {
-            float s = job.part[i];
-            for (uint32_t k = 1; k < job.ksplit; k++) s += job.part[(size_t)k * total + i];
-            job.y[i] = s;
-        }
-    }
+    if ((total & 3) == 0 && (reinterpret_cast<uintptr_t>(job.y) & 15) == 0)
+        mm_reduce_span(reinterpret_cast<const float4 *>(job.part), reinterpret_cast<float4 *>(job.y), total / 4, job.ksplit,
+                       first, stride);
+    else
+        mm_reduce_span(job.part, job.y, total, job.ksplit, first, stride);
 }
 
 // ------------------------------------------------------------------ launchers
@@ -1834,7 +2068,8 @@ static hipError_t launch_gemv_q4k(hipStream_t stream, const MatView *mats, float
     for (uint32_t j = n_jobs; j < GEMV_MAX_JOBS; j++) b.job[j] = b.job[0];
     b.total_rgs = rgs;
     const size_t lds = (size_t)n_iter * (64 * (lb * 4 + 4) + lb * 8) * sizeof(float);
-    if (lds > g_lds_limit) return hipErrorInvalidValue;
+    // rows of more than 64 super-blocks would need their two x regions in LDS at once (130 KB)
+    if (n_iter > 1 || lds > g_lds_limit) return hipErrorInvalidValue;
     const uint32_t units = rgs * n_iter;
     switch (lb) {
     // Short rows: small workgroups, so that even a 1024-row matrix spreads over every CU.
@@ -1890,7 +2125,7 @@ static hipError_t launch_gemv_q6k(hipStream_t stream, const MatView *mats, float
     for (uint32_t j = n_jobs; j < GEMV_MAX_JOBS; j++) b.job[j] = b.job[0];
     b.total_rgs = rgs;
     const size_t lds = (size_t)n_iter * (64 * (lb * 4 + 4) + lb * 16) * sizeof(float);
-    if (lds > g_lds_limit) return hipErrorInvalidValue;
+    if (n_iter > 1 || lds > g_lds_limit) return hipErrorInvalidValue;
     const uint32_t units = rgs * n_iter;
     switch (lb) {
     case 1: return launch_q6k_lb<1, 4>(stream, b, units, lds);
@@ -1900,6 +2135,71 @@ static hipError_t launch_gemv_q6k(hipStream_t stream, const MatView *mats, float
     case 16: return launch_q6k_lb<16, 4>(stream, b, units, lds);
     case 32: return launch_q6k_lb<32, 8>(stream, b, units, lds);
     default: return launch_q6k_lb<64, 8>(stream, b, units, lds);
+    }
+}
+
+template <uint32_t T, int LB, int NW>
+static hipError_t launch_b32_lb(hipStream_t stream, const GemvBatch &b, uint32_t units, size_t lds) {
+    const bool fp8 = T == T_Q4_0 && g_nib_mul != 0.f;
+    const void *kern = fp8 ? reinterpret_cast<const void *>(gemv_b32_kernel<T, LB, NW, true>)
+                           : reinterpret_cast<const void *>(gemv_b32_kernel<T, LB, NW, false>);
+    static size_t configured[2] = {0, 0};
+    if (lds > 48 * 1024 && lds > configured[fp8]) {
+        hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g_lds_limit);
+        if (e != hipSuccess) return e;
+        configured[fp8] = g_lds_limit;
+    }
+    size_t per_cu = g_lds_limit * 2 / (lds ? lds : 1);  // 160 KB of LDS per CU
+    if (per_cu < 1) per_cu = 1;
+    if (per_cu > 16 / NW) per_cu = 16 / NW;             // 16 wavefronts per CU
+    uint32_t grid = (uint32_t)((size_t)g_cu_count * per_cu);
+    const uint32_t needed = (units + NW - 1) / NW;
+    if (grid > needed) grid = needed;
+    const float mul = fp8 ? g_nib_mul : 1.0f, unit = fp8 ? 1.0f / g_nib_mul : 1.0f;
+    if (fp8)
+        hipLaunchKernelGGL((gemv_b32_kernel<T, LB, NW, true>), dim3(grid), dim3(NW * 64), lds, stream, b, mul, unit);
+    else
+        hipLaunchKernelGGL((gemv_b32_kernel<T, LB, NW, false>), dim3(grid), dim3(NW * 64), lds, stream, b, mul, unit);
+    return hipGetLastError();
+}
+
+// hipErrorInvalidValue: rows are not whole units (block-order layout) or x does not fit LDS.
+template <uint32_t T>
+static hipError_t launch_gemv_b32(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n_jobs,
+                                  const float *x) {
+    using G = B32Geo<T>;
+    const uint32_t cols = mats[0].cols;
+    if (!piece_major(T, cols)) return hipErrorInvalidValue;
+    const uint32_t nu = cols / G::UC;
+    uint32_t lb = 1;
+    while (lb < 64 && lb < nu) lb <<= 1;
+    const uint32_t rg_rows = 64 / lb, n_iter = (nu + lb - 1) / lb;
+    GemvBatch b;
+    b.x = x;
+    b.n_jobs = n_jobs;
+    b.n_chunks = nu * 8;
+    b.x_pad = cols;
+    uint32_t rgs = 0;
+    for (uint32_t j = 0; j < n_jobs; j++) {
+        b.job[j].m = mats[j];
+        b.job[j].y = ys[j];
+        b.job[j].rg_begin = rgs;
+        b.job[j].pad = 0;
+        rgs += (mats[j].rows + rg_rows - 1) / rg_rows;
+    }
+    for (uint32_t j = n_jobs; j < GEMV_MAX_JOBS; j++) b.job[j] = b.job[0];
+    b.total_rgs = rgs;
+    const size_t lds = (size_t)n_iter * ((G::UC / 4) * (lb * 4 + 4) + G::NBLK * lb) * sizeof(float);
+    if (lds > g_lds_limit) return hipErrorInvalidValue;
+    const uint32_t units = rgs;  // a wavefront keeps a row group for all of its n_iter unit columns
+    switch (lb) {
+    case 1: return launch_b32_lb<T, 1, 4>(stream, b, units, lds);
+    case 2: return launch_b32_lb<T, 2, 4>(stream, b, units, lds);
+    case 4: return launch_b32_lb<T, 4, 4>(stream, b, units, lds);
+    case 8: return launch_b32_lb<T, 8, 4>(stream, b, units, lds);
+    case 16: return launch_b32_lb<T, 16, 4>(stream, b, units, lds);
+    case 32: return launch_b32_lb<T, 32, 8>(stream, b, units, lds);
+    default: return launch_b32_lb<T, 64, 8>(stream, b, units, lds);
     }
 }
 
@@ -1914,6 +2214,11 @@ template <uint32_t T>
 static hipError_t launch_multi_t(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x) {
     if constexpr (T == T_Q4_K) return launch_gemv_q4k(stream, mats, ys, n, x);
     if constexpr (T == T_Q6_K) return launch_gemv_q6k(stream, mats, ys, n, x);
+    if constexpr (T == T_Q8_0 || T == T_Q4_0 || T == T_Q5_0 || T == T_Q5_1) {
+        hipError_t e = launch_gemv_b32<T>(stream, mats, ys, n, x);
+        if (e != hipErrorInvalidValue) return e;
+        (void)hipGetLastError();
+    }
     return launch_gemv_t<T, 4>(stream, mats, ys, n, x);
 }
 
@@ -1954,7 +2259,7 @@ static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *co
         // The column split of a product depends on that product alone, so that its
         // result does not change with what else shares the launch.
         const uint32_t tiles = job.tok_tiles * ((mats[j].rows + MM_ROWS - 1) / MM_ROWS);
-        uint32_t ks = (uint32_t)(2 * g_cu_count) / tiles;  // two workgroups per CU
+        uint32_t ks = (uint32_t)(2 * g_cu_count) / tiles;  // two workgroups per CU (measured best of 1..4)
         if (ks > n_steps / 8) ks = n_steps / 8;            // shares are whole 256-column units
         if (ks > 32) ks = 32;
         if (ks < 1) ks = 1;

@@ -16,9 +16,16 @@
 //   F16 / F32 : the row itself, zero-padded to a multiple of 8 elements
 //
 // Nothing is expanded: the planes hold exactly the bytes of the GGUF blocks
-// (F16/F32 rows gain at most 7 elements of zero padding), every code plane row
-// starts 16-byte aligned, and a wavefront's 64 x 16-byte load is one contiguous
-// kilobyte of a single row.
+// (F16/F32 rows gain at most 7 elements of zero padding) and every code plane
+// row starts 16-byte aligned.
+//
+// Code planes are stored piece-major.  The single-token kernels give one lane a
+// "unit" of a row (a 256-column super-block; 8 consecutive blocks of Q4_0/Q5_x;
+// 4 of Q8_0) whose codes are 8 pieces of 16 bytes (4 pieces for Q6_K's qh).
+// Piece cc of unit u of a row is stored at slot cc * units_per_row + u, so that
+// the lanes of a wavefront, which hold consecutive units and all fetch piece cc
+// at the same time, read one contiguous run.  Rows of the 32-column dtypes whose
+// length is not a whole number of units keep the block order (piece_major()).
 #pragma once
 #include <stddef.h>
 #include <stdint.h>
@@ -79,6 +86,32 @@ inline size_t gguf_row_bytes(uint32_t t, size_t cols) {
     size_t nb = cols / qk;
     if (nb != 0 && bb > SIZE_MAX / nb) return 0;
     return nb * bb;
+}
+
+#if defined(__HIPCC__)
+#define NH_HD __host__ __device__
+#else
+#define NH_HD
+#endif
+
+// Columns of the unit one lane of the single-token kernels owns.
+NH_HD inline uint32_t unit_cols(uint32_t t) { return t == T_Q8_0 ? 128u : 256u; }
+// Whether the code plane(s) of a matrix of this dtype and row length are piece-major.
+NH_HD inline bool piece_major(uint32_t t, size_t cols) {
+    switch (t) {
+    case T_Q4_K:
+    case T_Q6_K: return true;
+    case T_Q4_0:
+    case T_Q5_0:
+    case T_Q5_1:
+    case T_Q8_0: return cols % unit_cols(t) == 0;
+    default: return false;
+    }
+}
+// Byte offset, inside a row of a code plane with 8 pieces per unit, of the 16-byte piece that is
+// number `piece` of the row in block order.
+NH_HD inline size_t piece_offset(bool major, size_t units_per_row, size_t piece) {
+    return major ? ((piece & 7) * units_per_row + (piece >> 3)) * 16 : piece * 16;
 }
 
 struct PlaneSpec {
