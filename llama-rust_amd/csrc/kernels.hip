@@ -506,6 +506,9 @@ struct GemvBatch {
     GemvJob job[GEMV_MAX_JOBS];
     const float *x;
     uint32_t n_jobs, total_rgs, n_chunks, x_pad;
+    // Column window of the lane-per-unit kernels: units [unit0, unit0 + units) of every row.
+    // Rows too long for LDS are done in several launches, the later ones adding to y.
+    uint32_t unit0, units, accumulate, pad;
 };
 
 template <uint32_t T> __device__ __forceinline__ void load_x_lds(const float *xs, const float *sums, uint32_t c,
@@ -528,9 +531,13 @@ template <uint32_t T> __device__ __forceinline__ void load_x_lds(const float *xs
             o.x[4 * i] = a.x; o.x[4 * i + 1] = a.y; o.x[4 * i + 2] = a.z; o.x[4 * i + 3] = a.w;
         }
     }
-    float2 sm = *reinterpret_cast<const float2 *>(sums + 2 * c);
-    o.s_lo = sm.x;
-    o.s_hi = sm.y;
+    if constexpr (T == T_F32 || T == T_F16) {  // no code bias, no sums kept
+        o.s_lo = o.s_hi = 0.f;
+    } else {
+        float2 sm = *reinterpret_cast<const float2 *>(sums + 2 * c);
+        o.s_lo = sm.x;
+        o.s_hi = sm.y;
+    }
 }
 
 // Sum over the 64 lanes, valid in lane 63.  Four DPP steps inside each row of 16
@@ -588,7 +595,7 @@ __global__ __launch_bounds__(GEMV_WAVES * 64, 4) void gemv_kernel(const GemvBatc
 
     for (uint32_t i = tid; i < b.x_pad; i += GEMV_WAVES * 64) xs[i] = i < cols ? b.x[i] : 0.f;
     __syncthreads();
-    for (uint32_t c = tid; c < b.n_chunks; c += GEMV_WAVES * 64) {
+    for (uint32_t c = tid; c < (T == T_F32 || T == T_F16 ? 0u : b.n_chunks); c += GEMV_WAVES * 64) {
         float lo = 0.f, hi = 0.f;
 #pragma unroll
         for (int i = 0; i < E / 2; i++) {
@@ -723,8 +730,10 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b,
     constexpr uint32_t XROW = LB * 4 + 4;
     constexpr uint32_t XS_FLOATS = 64 * XROW;  // x region of one block iteration
     extern __shared__ __align__(16) float lds[];
-    const uint32_t nb = b.job[0].m.nb, cols = b.job[0].m.cols;
-    const uint32_t n_iter = (nb + LB - 1) / LB;  // block iterations per row (1 unless nb > 64)
+    const uint32_t nb_all = b.job[0].m.nb;         // super-blocks per row: slot stride of the piece-major plane
+    const uint32_t nb = b.units, cols = nb * 256;  // the window this launch covers
+    const float *xw = b.x + (size_t)b.unit0 * 256;
+    const uint32_t n_iter = (nb + LB - 1) / LB;    // always 1: the launcher cuts windows of at most 64 super-blocks
     // x, permuted so that lane blk reads piece i of code piece cc at a compile-time offset:
     //   float it * XS_FLOATS + (cc*8 + i) * XROW + (blk % LB) * 4 + e,   it = blk / LB
     float *xs = lds;
@@ -760,11 +769,11 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b,
         uint32_t row = w.row0 + sub_row;
         row = row < w.rows ? row : w.rows - 1;
         uint32_t blk = it * LB + b0;
-        blk = blk < nb ? blk : nb - 1;
+        blk = b.unit0 + (blk < nb ? blk : nb - 1);
         const uint32_t hoff = row * w.s1 + blk * 16, qoff = row * w.s0 + blk * 16;  // planes stay below 4 GB
         o.hdr = *reinterpret_cast<const uint4 *>(w.p1 + hoff);
 #pragma unroll
-        for (int cc = 0; cc < 8; cc++) o.q[cc] = *reinterpret_cast<const uint4 *>(w.p0 + (size_t)cc * nb * 16 + qoff);
+        for (int cc = 0; cc < 8; cc++) o.q[cc] = *reinterpret_cast<const uint4 *>(w.p0 + (size_t)cc * nb_all * 16 + qoff);
     };
 
     uint32_t u = blockIdx.x * GEMV_WAVES + wave;
@@ -792,7 +801,7 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b,
 #pragma unroll
         for (int k = 0; k < NXV; k++) {
             const uint32_t col = (tid + k * NW * 64) * 4;
-            xv[k] = *reinterpret_cast<const float4 *>(b.x + (col < cols ? col : 0));  // branch-free: stays first
+            xv[k] = *reinterpret_cast<const float4 *>(xw + (col < cols ? col : 0));  // branch-free: stays first
         }
         __builtin_amdgcn_sched_barrier(0);  // keep the x loads ahead of the weight loads in the queue
         fetch(u < n_units ? u : n_units - 1, ua);
@@ -807,7 +816,7 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b,
         NH_T(2);
     } else {
         for (uint32_t col = tid * 4; col < n_iter * LB * 256; col += NW * 64 * 4)
-            stage(col, col < cols ? *reinterpret_cast<const float4 *>(b.x + col) : make_float4(0.f, 0.f, 0.f, 0.f));
+            stage(col, col < cols ? *reinterpret_cast<const float4 *>(xw + col) : make_float4(0.f, 0.f, 0.f, 0.f));
         __syncthreads();
         if (u < n_units) fetch(u, ua);
     }
@@ -855,7 +864,7 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b,
             const Where w = locate(g);
             const float tot = group_sum_dpp<LB>(acc);
             const uint32_t row = w.row0 + sub_row;
-            if (b0 == LB - 1 && row < w.rows) w.y[row] = tot;
+            if (b0 == LB - 1 && row < w.rows) w.y[row] = b.accumulate ? w.y[row] + tot : tot;
             acc = 0.f;
         }
     };
@@ -898,7 +907,9 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q6k_kernel(const GemvBatch b)
     constexpr uint32_t XROW = LB * 4 + 4;
     constexpr uint32_t XS_FLOATS = 64 * XROW;
     extern __shared__ __align__(16) float lds[];
-    const uint32_t nb = b.job[0].m.nb, cols = b.job[0].m.cols;
+    const uint32_t nb_all = b.job[0].m.nb;         // super-blocks per row: slot stride of the piece-major planes
+    const uint32_t nb = b.units, cols = nb * 256;  // the window this launch covers
+    const float *xw = b.x + (size_t)b.unit0 * 256;
     const uint32_t n_iter = (nb + LB - 1) / LB;
     float *xs = lds;                                  // as in the Q4_K kernel, with this dtype's column order
     float *ssum = lds + (size_t)n_iter * XS_FLOATS;   // [it][16 column groups][blk % LB]
@@ -931,13 +942,13 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q6k_kernel(const GemvBatch b)
         uint32_t row = w.row0 + sub_row;
         row = row < w.rows ? row : w.rows - 1;
         uint32_t blk = it * LB + b0;
-        blk = blk < nb ? blk : nb - 1;
+        blk = b.unit0 + (blk < nb ? blk : nb - 1);
         const uint8_t *ql = w.p0 + (size_t)row * w.s0 + (size_t)blk * 16;
         const uint8_t *qh = w.p1 + (size_t)row * w.s1 + (size_t)blk * 16;
 #pragma unroll
-        for (int cc = 0; cc < 8; cc++) o.ql[cc] = *reinterpret_cast<const uint4 *>(ql + (size_t)cc * nb * 16);
+        for (int cc = 0; cc < 8; cc++) o.ql[cc] = *reinterpret_cast<const uint4 *>(ql + (size_t)cc * nb_all * 16);
 #pragma unroll
-        for (int hc = 0; hc < 4; hc++) o.qh[hc] = *reinterpret_cast<const uint4 *>(qh + (size_t)hc * nb * 16);
+        for (int hc = 0; hc < 4; hc++) o.qh[hc] = *reinterpret_cast<const uint4 *>(qh + (size_t)hc * nb_all * 16);
         o.sc = *reinterpret_cast<const uint4 *>(w.p2 + (size_t)row * w.s2 + (size_t)blk * 16);
         o.d = *reinterpret_cast<const uint16_t *>(w.p3 + (size_t)row * w.s3 + (size_t)blk * 2);
     };
@@ -954,7 +965,7 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q6k_kernel(const GemvBatch b)
         if ((lane & 3u) == 0) ssum[(it * 16 + (r >> 4)) * LB + bl] = sm;
     };
     for (uint32_t col = tid * 4; col < n_iter * LB * 256; col += NW * 64 * 4)
-        stage(col, *reinterpret_cast<const float4 *>(b.x + (col < cols ? col : 0)) );
+        stage(col, *reinterpret_cast<const float4 *>(xw + (col < cols ? col : 0)));
     __syncthreads();
 
     float acc = 0.f;
@@ -1008,7 +1019,7 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q6k_kernel(const GemvBatch b)
             const Where w = locate(g);
             const float tot = group_sum_dpp<LB>(acc);
             const uint32_t row = w.row0 + sub_row;
-            if (b0 == LB - 1 && row < w.rows) w.y[row] = tot;
+            if (b0 == LB - 1 && row < w.rows) w.y[row] = b.accumulate ? w.y[row] + tot : tot;
             acc = 0.f;
         }
     }
@@ -1043,8 +1054,9 @@ __global__ __launch_bounds__(NW * 64, (T == T_Q5_0 || T == T_Q5_1) ? 3 : 4) void
     constexpr uint32_t XROW = LB * 4 + 4;      // floats per LDS row: LB float4 plus one of padding
     constexpr uint32_t XS_FLOATS = (G::UC / 4) * XROW;
     extern __shared__ __align__(16) float lds[];
-    const uint32_t cols = b.job[0].m.cols;
-    const uint32_t nu = cols / G::UC;                 // units per row
+    const uint32_t nu_all = b.job[0].m.cols / G::UC;  // units per row: slot stride of the piece-major plane
+    const uint32_t nu = b.units, cols = nu * G::UC;   // the window this launch covers
+    const float *xw = b.x + (size_t)b.unit0 * G::UC;
     const uint32_t n_iter = (nu + LB - 1) / LB;
     float *xs = lds;                                   // [it][column / 4 of the unit][unit % LB] float4
     float *ssum = lds + (size_t)n_iter * XS_FLOATS;    // [it][block of the unit][unit % LB]: sum of x over the block
@@ -1089,10 +1101,10 @@ __global__ __launch_bounds__(NW * 64, (T == T_Q5_0 || T == T_Q5_1) ? 3 : 4) void
         uint32_t row = w.row0 + sub_row;
         row = row < m.rows ? row : m.rows - 1;
         uint32_t un = it * LB + b0;
-        un = un < nu ? un : nu - 1;
+        un = b.unit0 + (un < nu ? un : nu - 1);
         const uint8_t *q = m.p0 + (size_t)row * m.s0 + (size_t)un * 16;
 #pragma unroll
-        for (int cc = 0; cc < 8; cc++) o.q[cc] = *reinterpret_cast<const uint4 *>(q + (size_t)cc * nu * 16);
+        for (int cc = 0; cc < 8; cc++) o.q[cc] = *reinterpret_cast<const uint4 *>(q + (size_t)cc * nu_all * 16);
         if constexpr (T == T_Q8_0) {
             o.d = *reinterpret_cast<const uint2 *>(m.p1 + (size_t)row * m.s1 + (size_t)un * 8);
         } else if constexpr (T == T_Q4_0) {
@@ -1131,7 +1143,7 @@ __global__ __launch_bounds__(NW * 64, (T == T_Q5_0 || T == T_Q5_1) ? 3 : 4) void
 #pragma unroll
         for (int k = 0; k < NXV; k++) {
             const uint32_t col = (tid + k * NW * 64) * 4;
-            xv[k] = *reinterpret_cast<const float4 *>(b.x + (col < cols ? col : 0));  // branch-free: stays first
+            xv[k] = *reinterpret_cast<const float4 *>(xw + (col < cols ? col : 0));  // branch-free: stays first
         }
         __builtin_amdgcn_sched_barrier(0);  // keep the x loads ahead of the weight loads in the queue
         fetch(pa, ua);
@@ -1144,7 +1156,7 @@ __global__ __launch_bounds__(NW * 64, (T == T_Q5_0 || T == T_Q5_1) ? 3 : 4) void
         __syncthreads();
     } else {
         for (uint32_t col = tid * 4; col < n_iter * LB * G::UC; col += NW * 64 * 4)
-            stage(col, col < cols ? *reinterpret_cast<const float4 *>(b.x + col) : make_float4(0.f, 0.f, 0.f, 0.f));
+            stage(col, col < cols ? *reinterpret_cast<const float4 *>(xw + col) : make_float4(0.f, 0.f, 0.f, 0.f));
         __syncthreads();
         if (valid(pa)) fetch(pa, ua);
     }
@@ -1217,7 +1229,7 @@ __global__ __launch_bounds__(NW * 64, (T == T_Q5_0 || T == T_Q5_1) ? 3 : 4) void
             const Where w = locate(g);
             const float tot = group_sum_dpp<LB>(acc);
             const uint32_t row = w.row0 + sub_row;
-            if (b0 == LB - 1 && row < w.m->rows) w.y[row] = tot;
+            if (b0 == LB - 1 && row < w.m->rows) w.y[row] = b.accumulate ? w.y[row] + tot : tot;
             acc = 0.f;
         }
     };
@@ -1964,7 +1976,8 @@ static hipError_t launch_gemv_t(hipStream_t stream, const MatView *mats, float *
     }
     for (uint32_t j = n_jobs; j < GEMV_MAX_JOBS; j++) b.job[j] = b.job[0];
     b.total_rgs = rgs;
-    const size_t lds = ((size_t)b.x_pad + 2 * (size_t)b.n_chunks) * sizeof(float);
+    b.unit0 = b.units = b.accumulate = b.pad = 0;  // column windows are a lane-per-unit matter
+    const size_t lds = ((size_t)b.x_pad + (T == T_F32 || T == T_F16 ? 0 : 2 * (size_t)b.n_chunks)) * sizeof(float);
     if (lds > g_lds_limit) return hipErrorInvalidValue;
     auto kern = gemv_kernel<T, R>;
     static size_t configured = 0;  // per instantiation
@@ -2046,17 +2059,15 @@ static hipError_t launch_q4k_lb(hipStream_t stream, const GemvBatch &b, uint32_t
     return hipGetLastError();
 }
 
-static hipError_t launch_gemv_q4k(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n_jobs,
-                                  const float *x) {
-    const uint32_t nb = mats[0].nb;
-    uint32_t lb = 1;
-    while (lb < 64 && lb < nb) lb <<= 1;
-    const uint32_t rg_rows = 64 / lb, n_iter = (nb + lb - 1) / lb;
-    GemvBatch b;
+// Jobs of a lane-per-unit launch: lb lanes per row, 64 / lb rows per wavefront step.
+static uint32_t fill_unit_jobs(GemvBatch &b, const MatView *mats, float *const *ys, uint32_t n_jobs, const float *x,
+                               uint32_t lb) {
+    const uint32_t rg_rows = 64 / lb;
     b.x = x;
     b.n_jobs = n_jobs;
-    b.n_chunks = nb * 8;
+    b.n_chunks = 0;
     b.x_pad = mats[0].cols;
+    b.pad = 0;
     uint32_t rgs = 0;
     for (uint32_t j = 0; j < n_jobs; j++) {
         b.job[j].m = mats[j];
@@ -2067,20 +2078,48 @@ static hipError_t launch_gemv_q4k(hipStream_t stream, const MatView *mats, float
     }
     for (uint32_t j = n_jobs; j < GEMV_MAX_JOBS; j++) b.job[j] = b.job[0];
     b.total_rgs = rgs;
-    const size_t lds = (size_t)n_iter * (64 * (lb * 4 + 4) + lb * 8) * sizeof(float);
-    // rows of more than 64 super-blocks would need their two x regions in LDS at once (130 KB)
-    if (n_iter > 1 || lds > g_lds_limit) return hipErrorInvalidValue;
-    const uint32_t units = rgs * n_iter;
-    switch (lb) {
-    // Short rows: small workgroups, so that even a 1024-row matrix spreads over every CU.
-    case 1: return launch_q4k_lb<1, 4>(stream, b, units, lds);
-    case 2: return launch_q4k_lb<2, 4>(stream, b, units, lds);
-    case 4: return launch_q4k_lb<4, 4>(stream, b, units, lds);
-    case 8: return launch_q4k_lb<8, 4>(stream, b, units, lds);
-    case 16: return launch_q4k_lb<16, 4>(stream, b, units, lds);
-    case 32: return launch_q4k_lb<32, 8>(stream, b, units, lds);
-    default: return launch_q4k_lb<64, 8>(stream, b, units, lds);
+    return rgs;
+}
+
+// Rows of nu units are cut into the fewest equal windows of at most max_units; window w
+// covers units [first, first + count).
+struct UnitWindows {
+    uint32_t n, per;
+    UnitWindows(uint32_t nu, uint32_t max_units) : n((nu + max_units - 1) / max_units), per((nu + n - 1) / n) {}
+    uint32_t first(uint32_t w) const { return w * per; }
+    uint32_t count(uint32_t w, uint32_t nu) const { return first(w) + per <= nu ? per : nu - first(w); }
+};
+
+static hipError_t launch_gemv_q4k(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n_jobs,
+                                  const float *x) {
+    const uint32_t nb = mats[0].nb;
+    // one lane per super-block, at most 64 per row and launch: longer rows take several launches
+    const UnitWindows win(nb, 64);
+    for (uint32_t w = 0; w < win.n; w++) {
+        const uint32_t units = win.count(w, nb);
+        uint32_t lb = 1;
+        while (lb < 64 && lb < units) lb <<= 1;
+        GemvBatch b;
+        const uint32_t rgs = fill_unit_jobs(b, mats, ys, n_jobs, x, lb);
+        b.unit0 = win.first(w);
+        b.units = units;
+        b.accumulate = w > 0;
+        const size_t lds = (size_t)(64 * (lb * 4 + 4) + lb * 8) * sizeof(float);
+        if (lds > g_lds_limit) return hipErrorInvalidValue;
+        hipError_t e;
+        switch (lb) {
+        // Short rows: small workgroups, so that even a 1024-row matrix spreads over every CU.
+        case 1: e = launch_q4k_lb<1, 4>(stream, b, rgs, lds); break;
+        case 2: e = launch_q4k_lb<2, 4>(stream, b, rgs, lds); break;
+        case 4: e = launch_q4k_lb<4, 4>(stream, b, rgs, lds); break;
+        case 8: e = launch_q4k_lb<8, 4>(stream, b, rgs, lds); break;
+        case 16: e = launch_q4k_lb<16, 4>(stream, b, rgs, lds); break;
+        case 32: e = launch_q4k_lb<32, 8>(stream, b, rgs, lds); break;
+        default: e = launch_q4k_lb<64, 8>(stream, b, rgs, lds); break;
+        }
+        if (e != hipSuccess) return e;
     }
+    return hipSuccess;
 }
 
 template <int LB, int NW>
@@ -2106,36 +2145,31 @@ static hipError_t launch_q6k_lb(hipStream_t stream, const GemvBatch &b, uint32_t
 static hipError_t launch_gemv_q6k(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n_jobs,
                                   const float *x) {
     const uint32_t nb = mats[0].nb;
-    uint32_t lb = 1;
-    while (lb < 64 && lb < nb) lb <<= 1;
-    const uint32_t rg_rows = 64 / lb, n_iter = (nb + lb - 1) / lb;
-    GemvBatch b;
-    b.x = x;
-    b.n_jobs = n_jobs;
-    b.n_chunks = nb * 8;
-    b.x_pad = mats[0].cols;
-    uint32_t rgs = 0;
-    for (uint32_t j = 0; j < n_jobs; j++) {
-        b.job[j].m = mats[j];
-        b.job[j].y = ys[j];
-        b.job[j].rg_begin = rgs;
-        b.job[j].pad = 0;
-        rgs += (mats[j].rows + rg_rows - 1) / rg_rows;
+    const UnitWindows win(nb, 64);
+    for (uint32_t w = 0; w < win.n; w++) {
+        const uint32_t units = win.count(w, nb);
+        uint32_t lb = 1;
+        while (lb < 64 && lb < units) lb <<= 1;
+        GemvBatch b;
+        const uint32_t rgs = fill_unit_jobs(b, mats, ys, n_jobs, x, lb);
+        b.unit0 = win.first(w);
+        b.units = units;
+        b.accumulate = w > 0;
+        const size_t lds = (size_t)(64 * (lb * 4 + 4) + lb * 16) * sizeof(float);
+        if (lds > g_lds_limit) return hipErrorInvalidValue;
+        hipError_t e;
+        switch (lb) {
+        case 1: e = launch_q6k_lb<1, 4>(stream, b, rgs, lds); break;
+        case 2: e = launch_q6k_lb<2, 4>(stream, b, rgs, lds); break;
+        case 4: e = launch_q6k_lb<4, 4>(stream, b, rgs, lds); break;
+        case 8: e = launch_q6k_lb<8, 4>(stream, b, rgs, lds); break;
+        case 16: e = launch_q6k_lb<16, 4>(stream, b, rgs, lds); break;
+        case 32: e = launch_q6k_lb<32, 8>(stream, b, rgs, lds); break;
+        default: e = launch_q6k_lb<64, 8>(stream, b, rgs, lds); break;
+        }
+        if (e != hipSuccess) return e;
     }
-    for (uint32_t j = n_jobs; j < GEMV_MAX_JOBS; j++) b.job[j] = b.job[0];
-    b.total_rgs = rgs;
-    const size_t lds = (size_t)n_iter * (64 * (lb * 4 + 4) + lb * 16) * sizeof(float);
-    if (n_iter > 1 || lds > g_lds_limit) return hipErrorInvalidValue;
-    const uint32_t units = rgs * n_iter;
-    switch (lb) {
-    case 1: return launch_q6k_lb<1, 4>(stream, b, units, lds);
-    case 2: return launch_q6k_lb<2, 4>(stream, b, units, lds);
-    case 4: return launch_q6k_lb<4, 4>(stream, b, units, lds);
-    case 8: return launch_q6k_lb<8, 4>(stream, b, units, lds);
-    case 16: return launch_q6k_lb<16, 4>(stream, b, units, lds);
-    case 32: return launch_q6k_lb<32, 8>(stream, b, units, lds);
-    default: return launch_q6k_lb<64, 8>(stream, b, units, lds);
-    }
+    return hipSuccess;
 }
 
 template <uint32_t T, int LB, int NW>
@@ -2163,7 +2197,7 @@ static hipError_t launch_b32_lb(hipStream_t stream, const GemvBatch &b, uint32_t
     return hipGetLastError();
 }
 
-// hipErrorInvalidValue: rows are not whole units (block-order layout) or x does not fit LDS.
+// hipErrorInvalidValue: rows are not whole units (block-order layout).
 template <uint32_t T>
 static hipError_t launch_gemv_b32(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n_jobs,
                                   const float *x) {
@@ -2171,36 +2205,35 @@ static hipError_t launch_gemv_b32(hipStream_t stream, const MatView *mats, float
     const uint32_t cols = mats[0].cols;
     if (!piece_major(T, cols)) return hipErrorInvalidValue;
     const uint32_t nu = cols / G::UC;
-    uint32_t lb = 1;
-    while (lb < 64 && lb < nu) lb <<= 1;
-    const uint32_t rg_rows = 64 / lb, n_iter = (nu + lb - 1) / lb;
-    GemvBatch b;
-    b.x = x;
-    b.n_jobs = n_jobs;
-    b.n_chunks = nu * 8;
-    b.x_pad = cols;
-    uint32_t rgs = 0;
-    for (uint32_t j = 0; j < n_jobs; j++) {
-        b.job[j].m = mats[j];
-        b.job[j].y = ys[j];
-        b.job[j].rg_begin = rgs;
-        b.job[j].pad = 0;
-        rgs += (mats[j].rows + rg_rows - 1) / rg_rows;
+    // up to 64 lanes per row, and as many unit columns per lane as keep x within LDS
+    const size_t iter_lds = (size_t)((G::UC / 4) * (64 * 4 + 4) + G::NBLK * 64) * sizeof(float);
+    const uint32_t max_iter = (uint32_t)(g_lds_limit / iter_lds) ? (uint32_t)(g_lds_limit / iter_lds) : 1;
+    const UnitWindows win(nu, 64 * max_iter);
+    for (uint32_t w = 0; w < win.n; w++) {
+        const uint32_t units = win.count(w, nu);
+        uint32_t lb = 1;
+        while (lb < 64 && lb < units) lb <<= 1;
+        const uint32_t n_iter = (units + lb - 1) / lb;
+        GemvBatch b;
+        const uint32_t rgs = fill_unit_jobs(b, mats, ys, n_jobs, x, lb);
+        b.unit0 = win.first(w);
+        b.units = units;
+        b.accumulate = w > 0;
+        const size_t lds = (size_t)n_iter * ((G::UC / 4) * (lb * 4 + 4) + G::NBLK * lb) * sizeof(float);
+        if (lds > g_lds_limit) return hipErrorInvalidValue;
+        hipError_t e;
+        switch (lb) {
+        case 1: e = launch_b32_lb<T, 1, 4>(stream, b, rgs, lds); break;
+        case 2: e = launch_b32_lb<T, 2, 4>(stream, b, rgs, lds); break;
+        case 4: e = launch_b32_lb<T, 4, 4>(stream, b, rgs, lds); break;
+        case 8: e = launch_b32_lb<T, 8, 4>(stream, b, rgs, lds); break;
+        case 16: e = launch_b32_lb<T, 16, 4>(stream, b, rgs, lds); break;
+        case 32: e = launch_b32_lb<T, 32, 8>(stream, b, rgs, lds); break;
+        default: e = launch_b32_lb<T, 64, 8>(stream, b, rgs, lds); break;
+        }
+        if (e != hipSuccess) return e;
     }
-    for (uint32_t j = n_jobs; j < GEMV_MAX_JOBS; j++) b.job[j] = b.job[0];
-    b.total_rgs = rgs;
-    const size_t lds = (size_t)n_iter * ((G::UC / 4) * (lb * 4 + 4) + G::NBLK * lb) * sizeof(float);
-    if (lds > g_lds_limit) return hipErrorInvalidValue;
-    const uint32_t units = rgs;  // a wavefront keeps a row group for all of its n_iter unit columns
-    switch (lb) {
-    case 1: return launch_b32_lb<T, 1, 4>(stream, b, units, lds);
-    case 2: return launch_b32_lb<T, 2, 4>(stream, b, units, lds);
-    case 4: return launch_b32_lb<T, 4, 4>(stream, b, units, lds);
-    case 8: return launch_b32_lb<T, 8, 4>(stream, b, units, lds);
-    case 16: return launch_b32_lb<T, 16, 4>(stream, b, units, lds);
-    case 32: return launch_b32_lb<T, 32, 8>(stream, b, units, lds);
-    default: return launch_b32_lb<T, 64, 8>(stream, b, units, lds);
-    }
+    return hipSuccess;
 }
 
 template <uint32_t T>

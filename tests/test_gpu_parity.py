@@ -194,9 +194,9 @@ def test_random_gemv_and_gemm_within_bounds(pkg, gpu, ty):
     if K.QK[ty] == 1:
         shapes = [(5, 1), (33, 7), (64, 100), (130, 257), (19, 1000), (300, 4096), (64, 4100)]
     elif K.QK[ty] == 32:
-        shapes = [(3, 32), (65, 64), (10, 96), (33, 2048), (257, 4096), (40, 14336), (16, 16416)]
+        shapes = [(3, 32), (65, 64), (10, 96), (33, 2048), (257, 4096), (40, 14336), (16, 16416), (6, 28672)]
     else:
-        shapes = [(3, 256), (65, 512), (9, 768), (33, 2048), (257, 4096), (40, 14336), (12, 16640)]
+        shapes = [(3, 256), (65, 512), (9, 768), (33, 2048), (257, 4096), (40, 14336), (12, 16640), (6, 28672)]
     for rows, cols in shapes:
         w = K.random_packed(ty, rows, cols, rng)
         m = gpu.upload_packed(ty, rows, cols, w)
