@@ -16,6 +16,13 @@ launch / mean launch duration from HIP events recorded on the launch stream
 around the Q4_K part of every timed step.  `cpu_baseline` times the AVX2 port of
 the reference's `simd` CPU kernels on a bounded sample of the same workload.
 
+`other_workloads` times, after the headline run and outside its timed region, the
+other shapes the reference's benchmarks name: the Q8_0 4096x4096 GEMV, the
+Q4_0 4096x14336 product at 8..512 tokens, and one Mixtral-shaped MoE projection
+(8 Q4_K experts, 16 tokens each) as a single grouped call.  Each figure is a
+mean over launches that rotate through enough distinct matrices to defeat the
+256 MB Infinity Cache, from HIP events on the launch stream.
+
 One JSON line on stdout; progress on stderr.
 """
 import argparse
@@ -32,7 +39,9 @@ sys.path.insert(0, ROOT)
 
 METRIC = "Q4_K/Q8_0 GEMV HBM GB/s (% of peak); 8B-shape decode tok/s, batch 1"
 HBM_PEAK_GBS = 8000.0
-Q4_K, Q6_K = 12, 14
+BF16_MFMA_PEAK_TFLOPS = 2500.0
+Q4_0, Q8_0, Q4_K, Q6_K = 2, 8, 12, 14
+BLOCK = {Q4_0: (32, 18, 0), Q8_0: (32, 34, 0), Q4_K: (256, 144, 0), Q6_K: (256, 210, 208)}  # columns, bytes, offset of d
 N_LAYERS, D, D_KV, FF, VOCAB = 32, 4096, 1024, 14336, 128256
 # (name, rows, cols, which activation buffer it reads).  Products that read the same buffer are
 # independent of each other (q/k/v of the normed hidden state, gate/up of the normed residual);
@@ -48,7 +57,8 @@ def log(*a):
 
 
 def row_bytes(ty, cols):
-    return cols // 256 * (144 if ty == Q4_K else 210)
+    qk, bb, _ = BLOCK[ty]
+    return cols // qk * bb
 
 
 def algorithmic_bytes(ty, rows, cols, tokens=1):
@@ -58,13 +68,12 @@ def algorithmic_bytes(ty, rows, cols, tokens=1):
 
 def synth_matrix(ty, rows, cols, rng):
     """Packed GGUF bytes: uniform random codes / 6-bit scales, |N(0, 0.02)| f16 super-block scales."""
-    nb = cols // 256
-    bb = 144 if ty == Q4_K else 210
+    qk, bb, d_off = BLOCK[ty]
+    nb = cols // qk
     blk = rng.integers(0, 256, size=(rows, nb, bb), dtype=np.uint8)
-    if ty == Q4_K:
-        blk[:, :, 0:4] = np.abs(rng.normal(0, 0.02, (rows, nb, 2))).astype(np.float16).view(np.uint8).reshape(rows, nb, 4)
-    else:
-        blk[:, :, 208:210] = np.abs(rng.normal(0, 0.02, (rows, nb, 1))).astype(np.float16).view(np.uint8).reshape(rows, nb, 2)
+    n_scales = 2 if ty == Q4_K else 1  # Q4_K: d and dmin
+    blk[:, :, d_off:d_off + 2 * n_scales] = (np.abs(rng.normal(0, 0.02, (rows, nb, n_scales))).astype(np.float16)
+                                             .view(np.uint8).reshape(rows, nb, 2 * n_scales))
     return blk.reshape(-1)
 
 
@@ -94,6 +103,87 @@ def cpu_baseline(sample, x_by_cols, seconds):
             "tok_per_s_equiv": n / dt * nbytes / TOKEN_BYTES}
 
 
+def timed_us(hip, stream, enqueue, n_variants, reps):
+    """Mean microseconds of enqueue(i), i rotating over n_variants, from HIP events on `stream`."""
+    for i in range(n_variants):
+        enqueue(i)
+    stream.synchronize()
+    a, b = hip.Event(), hip.Event()
+    a.record(stream)
+    for r in range(reps):
+        for i in range(n_variants):
+            enqueue(i)
+    b.record(stream)
+    stream.synchronize()
+    return a.elapsed_ms(b) * 1e3 / (reps * n_variants)
+
+
+def other_workloads(pkg, hip, gpu, stream, rng):
+    """Shapes of the reference's other benchmark configurations (see the module docstring)."""
+    import oracle as O
+    out = {}
+
+    def check(name, ty, rows, cols, tokens, w, x, y_dev):
+        got = y_dev.to_numpy(np.float32)[:tokens * rows].reshape(tokens, rows)[:, :32]
+        want = O.gemm_f64(ty, cols, tokens, w[:32 * row_bytes(ty, cols)], x, 32)
+        want = np.asarray(want).reshape(tokens, 32)
+        if not np.allclose(got, want, rtol=1e-4, atol=1e-4 * float(np.sqrt(np.mean(want ** 2)))):
+            raise RuntimeError(f"{name}: GPU output disagrees with the CPU oracle")
+
+    # Q8_0 4096x4096, one token (the reference's demo shape)
+    n = 16
+    ws = [synth_matrix(Q8_0, D, D, rng) for _ in range(n)]
+    ms = [gpu.upload_packed(Q8_0, D, D, w) for w in ws]
+    x = rng.normal(0, 1, D).astype(np.float32)
+    xd, yd = hip.DeviceBuffer.from_numpy(x), hip.DeviceBuffer(D * 4)
+    us = timed_us(hip, stream, lambda i: gpu.gemm_device(ms[i], 1, xd.ptr, yd.ptr, stream.ptr), n, 20)
+    gpu.gemm_device(ms[0], 1, xd.ptr, yd.ptr, stream.ptr); stream.synchronize()
+    check("Q8_0 GEMV", Q8_0, D, D, 1, ws[0], x, yd)
+    nbytes = algorithmic_bytes(Q8_0, D, D)
+    out["gemv_q8_0_4096x4096"] = {"launch_us": round(us, 2), "achieved": round(nbytes / us / 1e3, 1), "unit": "GB/s",
+                                  "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "bound": "hbm"}
+    for m in ms:
+        m.close()
+
+    # Q4_0 4096x14336 at 8..512 tokens (chunked prefill)
+    n = 8
+    ws = [synth_matrix(Q4_0, D, FF, rng) for _ in range(n)]
+    ms = [gpu.upload_packed(Q4_0, D, FF, w) for w in ws]
+    x = rng.normal(0, 1, 512 * FF).astype(np.float32)
+    xd, yd = hip.DeviceBuffer.from_numpy(x), hip.DeviceBuffer(512 * D * 4)
+    for tokens in (8, 32, 128, 512):
+        us = timed_us(hip, stream, lambda i: gpu.gemm_device(ms[i], tokens, xd.ptr, yd.ptr, stream.ptr), n, 5)
+        gpu.gemm_device(ms[0], tokens, xd.ptr, yd.ptr, stream.ptr); stream.synchronize()
+        check(f"Q4_0 GEMM M={tokens}", Q4_0, D, FF, tokens, ws[0], x[:tokens * FF], yd)
+        flops = 2.0 * D * FF * tokens
+        # three bf16 MFMA products per multiply-add (the f32 activations are split in three)
+        out[f"gemm_q4_0_4096x14336_m{tokens}"] = {
+            "call_us": round(us, 2), "tflops": round(flops / us / 1e6, 1),
+            "mfma_frac": round(3 * flops / us / 1e6 / BF16_MFMA_PEAK_TFLOPS, 4),
+            "weight_gbs": round(D * row_bytes(Q4_0, FF) / us / 1e3, 1), "bound": "mfma" if tokens >= 128 else "hbm"}
+    for m in ms:
+        m.close()
+
+    # one MoE projection: 8 Q4_K experts 4096 -> 14336, 16 tokens each, one grouped call
+    n_exp, per = 8, 16
+    sets = 2  # two sets of experts = 528 MB, so that no call is served from the Infinity Cache
+    ws = [[synth_matrix(Q4_K, FF, D, rng) for _ in range(n_exp)] for _ in range(sets)]
+    ms = [[gpu.upload_packed(Q4_K, FF, D, w) for w in ws_] for ws_ in ws]
+    x = rng.normal(0, 1, n_exp * per * D).astype(np.float32)
+    xd, yd = hip.DeviceBuffer.from_numpy(x), hip.DeviceBuffer(n_exp * per * FF * 4)
+    us = timed_us(hip, stream, lambda i: gpu.gemm_grouped_device(ms[i], [per] * n_exp, xd.ptr, yd.ptr, stream.ptr), sets, 10)
+    gpu.gemm_grouped_device(ms[0], [per] * n_exp, xd.ptr, yd.ptr, stream.ptr); stream.synchronize()
+    check("MoE grouped GEMM", Q4_K, FF, D, per, ws[0][0], x[:per * D], yd)
+    wbytes = n_exp * FF * row_bytes(Q4_K, D)
+    out["moe_q4_k_8x14336x4096_m16"] = {"call_us": round(us, 2), "weight_gbs": round(wbytes / us / 1e3, 1),
+                                         "frac": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                                         "tflops": round(2.0 * n_exp * per * FF * D / us / 1e6, 1), "bound": "hbm"}
+    for ms_ in ms:
+        for m in ms_:
+            m.close()
+    return out
+
+
 TOKEN_BYTES = N_LAYERS * sum(algorithmic_bytes(Q4_K, r, c) for _, r, c, _ in LAYER) + algorithmic_bytes(Q6_K, VOCAB, D)
 
 
@@ -106,6 +196,7 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="enqueue every product eagerly instead of replaying HIP graphs")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="0 skips the CPU baseline")
     ap.add_argument("--seed", type=int, default=20240531)
+    ap.add_argument("--no-extras", action="store_true", help="skip the other_workloads section")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB copy kernel three times (known traffic for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -222,10 +313,16 @@ def main():
                      "unit": "GB/s", "frac": round(q4k_gbs / HBM_PEAK_GBS, 4), "traffic": None,
                      "bytes_per_launch": round(q4k_bytes / n_launch), "launch_us": round(q4k_launch_us, 3),
                      "launches_timed": args.steps * n_launch},
-        "other_kernels": {"gemv_kernel<Q6_K> head": {"achieved": round(head_gbs, 1), "unit": "GB/s",
+        "other_kernels": {"gemv_q6k_kernel (head)": {"achieved": round(head_gbs, 1), "unit": "GB/s",
                                                      "frac": round(head_gbs / HBM_PEAK_GBS, 4),
                                                      "launch_us": round(head_ms * 1e3 / args.steps, 2)}},
     }
+    if not args.no_extras:
+        log("[bench] other workloads (Q8_0 GEMV, Q4_0 prefill GEMM, MoE grouped GEMM) ...")
+        for m in mats:
+            m.close()
+        head.close()
+        out["other_workloads"] = other_workloads(pkg, hip, gpu, stream, rng)
     if args.cpu_seconds > 0:
         log("[bench] timing the CPU baseline ...")
         out["cpu_baseline"] = cpu_baseline(sample, x_host, args.cpu_seconds)

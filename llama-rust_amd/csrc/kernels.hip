@@ -1453,6 +1453,7 @@ struct MmBatch {
     uint4 *xb;   // [group of 16 columns][part 0..2][half 0..1][token slot] x 8 bf16
     float *sx;   // [group of 16 columns][token slot]: sum of the group's activations
     uint32_t n_jobs, total_wgs, mpad, any_split;
+    uint32_t nibble_bf16, pad0, pad1, pad2;  // nibble_bf16: the device converts nibble bytes straight to bf16 integers
 };
 
 template <uint32_t T> struct MmTraits {
@@ -1556,11 +1557,12 @@ __device__ __forceinline__ void mm_codes4(uint32_t bytes, float bias, float *f) 
 
 // Codes of the two groups of step s as bf16 (frag[g][half]), with scale[g] and
 // offset[g]: W[row, col] = scale * code + offset.
-template <uint32_t T>
+template <uint32_t T, bool NIBBLE_BF16>
 __device__ __forceinline__ void mm_decode(const MmRaw<T> &raw, uint32_t s, uint4 (&frag)[2][2], float (&scale)[2],
                                           float (&offset)[2]) {
     float f[2][16];
     offset[0] = offset[1] = 0.f;
+    bool packed_done = false;  // frag already written by the fp8 -> bf16 path
     if constexpr (T == T_Q8_0) {
         const uint32_t w[8] = {raw.q0.x, raw.q0.y, raw.q0.z, raw.q0.w, raw.q1.x, raw.q1.y, raw.q1.z, raw.q1.w};
 #pragma unroll
@@ -1595,10 +1597,28 @@ __device__ __forceinline__ void mm_decode(const MmRaw<T> &raw, uint32_t s, uint4
     } else if constexpr (T == T_Q4_K) {
         const Raw<T> &r = raw.r;
         const uint32_t w[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+        if constexpr (NIBBLE_BF16) {  // one convert per two codes, no f32 in between
+            uint32_t o[2][8];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            mm_codes4(w[i] & 0x0f0f0f0fu, 0.f, f[0] + 4 * i);
-            mm_codes4((w[i] >> 4) & 0x0f0f0f0fu, 0.f, f[1] + 4 * i);
+            for (int i = 0; i < 4; i++) {
+                const uint32_t lo = w[i] & 0x0f0f0f0fu, hi = (w[i] >> 4) & 0x0f0f0f0fu;
+                o[0][2 * i] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)lo, 512.0f, false));
+                o[0][2 * i + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)lo, 512.0f, true));
+                o[1][2 * i] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)hi, 512.0f, false));
+                o[1][2 * i + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)hi, 512.0f, true));
+            }
+#pragma unroll
+            for (int g = 0; g < 2; g++) {
+                frag[g][0] = make_uint4(o[g][0], o[g][1], o[g][2], o[g][3]);
+                frag[g][1] = make_uint4(o[g][4], o[g][5], o[g][6], o[g][7]);
+            }
+            packed_done = true;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                mm_codes4(w[i] & 0x0f0f0f0fu, 0.f, f[0] + 4 * i);
+                mm_codes4((w[i] >> 4) & 0x0f0f0f0fu, 0.f, f[1] + 4 * i);
+            }
         }
         // 6-bit (scale, min) pairs 2g and 2g+1 of the block, g = (s % 8) / 2 (langtax/src/quant.rs:8901-8912)
         const uint32_t g = (s & 7u) >> 1;
@@ -1633,10 +1653,12 @@ __device__ __forceinline__ void mm_decode(const MmRaw<T> &raw, uint32_t s, uint4
         scale[0] = d * (float)(int)(int8_t)(r.sc.x >> sh);
         scale[1] = d * (float)(int)(int8_t)(r.sc.y >> sh);
     }
+    if (!packed_done) {
 #pragma unroll
-    for (int g = 0; g < 2; g++) {
-        frag[g][0] = bf16x8_of(f[g]);
-        frag[g][1] = bf16x8_of(f[g] + 8);
+        for (int g = 0; g < 2; g++) {
+            frag[g][0] = bf16x8_of(f[g]);
+            frag[g][1] = bf16x8_of(f[g] + 8);
+        }
     }
 }
 
@@ -1654,8 +1676,12 @@ template <uint32_t T, int TT> struct MmStage {
     static constexpr size_t BYTES = SX + (OFFSET ? (size_t)256 * 4 : 0);
 };
 
-template <uint32_t T, int TT>
+// TT: token tiles of 32 per workgroup.  VQ: how many of a tile's four 8-token quads can hold
+// tokens (a lane's accumulator v belongs to quad v / 4); the others are neither scaled nor stored.
+// FB: nibble bytes go straight to bf16 with the packed fp8 convert (Q4_K, when the device probe allows).
+template <uint32_t T, int TT, int VQ, bool FB>
 __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const MmBatch b) {
+    constexpr int NV = 4 * VQ;
     using St = MmStage<T, TT>;
     constexpr bool OFFSET = St::OFFSET;
     constexpr bool SAME_SCALE = MmTraits<T>::SAME_SCALE;
@@ -1740,7 +1766,7 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const MmBatch b) {
         uint8_t *st = mm_lds + (size_t)buf * St::BYTES;
         uint4 frag[2][2];
         float sc[2], of[2];
-        mm_decode<T>(raw, s, frag, sc, of);
+        mm_decode<T, FB>(raw, s, frag, sc, of);
         uint4 *code_s = reinterpret_cast<uint4 *>(st + St::CODE);
         float *scale_s = reinterpret_cast<float *>(st + St::SCALE);
 #pragma unroll
@@ -1794,7 +1820,7 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const MmBatch b) {
             // sxv: sums of activations (over the 32 columns an offset covers) of the lane's 16 token rows
             auto load_sx = [&](int g, float (&sxv)[16]) {
 #pragma unroll
-                for (int q = 0; q < 4; q++) {
+                for (int q = 0; q < VQ; q++) {
                     const float4 t4 = *reinterpret_cast<const float4 *>(sx_s + g * TOK + tt * 32 + 8 * q + 4 * kh);
                     sxv[4 * q] = t4.x; sxv[4 * q + 1] = t4.y; sxv[4 * q + 2] = t4.z; sxv[4 * q + 3] = t4.w;
                 }
@@ -1814,10 +1840,10 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const MmBatch b) {
                         p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[g][0], wf[g][rs], p, 0, 0, 0);
                     }
 #pragma unroll
-                    for (int v = 0; v < 16; v++) acc[rs][tt][v] = fmaf(sc[0][rs], p[v], acc[rs][tt][v]);
+                    for (int v = 0; v < NV; v++) acc[rs][tt][v] = fmaf(sc[0][rs], p[v], acc[rs][tt][v]);
                     if constexpr (with_offset) {
 #pragma unroll
-                        for (int v = 0; v < 16; v++) acc[rs][tt][v] = fmaf(of[0][rs], sxv[v], acc[rs][tt][v]);
+                        for (int v = 0; v < NV; v++) acc[rs][tt][v] = fmaf(of[0][rs], sxv[v], acc[rs][tt][v]);
                     }
                 }
             } else {
@@ -1834,10 +1860,10 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const MmBatch b) {
                         p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[g][1], wf[g][rs], p, 0, 0, 0);
                         p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[g][0], wf[g][rs], p, 0, 0, 0);
 #pragma unroll
-                        for (int v = 0; v < 16; v++) acc[rs][tt][v] = fmaf(sc[g][rs], p[v], acc[rs][tt][v]);
+                        for (int v = 0; v < NV; v++) acc[rs][tt][v] = fmaf(sc[g][rs], p[v], acc[rs][tt][v]);
                         if constexpr (with_offset) {
 #pragma unroll
-                            for (int v = 0; v < 16; v++) acc[rs][tt][v] = fmaf(of[g][rs], sxv[v], acc[rs][tt][v]);
+                            for (int v = 0; v < NV; v++) acc[rs][tt][v] = fmaf(of[g][rs], sxv[v], acc[rs][tt][v]);
                         }
                     }
                 }
@@ -1902,7 +1928,7 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const MmBatch b) {
 #pragma unroll
         for (int tt = 0; tt < TT; tt++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
+            for (int v = 0; v < NV; v++) {
                 const uint32_t t = tok0 + tt * 32 + 8 * (v >> 2) + 4 * kh + (v & 3);
                 if (t < job.tokens) out[(size_t)t * m.rows + row] = acc[rs][tt][v];
             }
@@ -1946,6 +1972,7 @@ __global__ __launch_bounds__(256) void mm_reduce_kernel(const MmBatch b) {
 
 // ------------------------------------------------------------------ launchers
 
+static bool g_nibble_bf16 = false;  // the packed fp8 -> bf16 convert turns nibble bytes into the integers 0..15
 static int g_cu_count = 256;
 static size_t g_lds_limit = 64 * 1024;
 
@@ -2006,14 +2033,23 @@ __global__ void fp8_nibble_probe(float *out) {
     out[4 * threadIdx.x + 1] = v[1];
     out[4 * threadIdx.x + 2] = w[0];
     out[4 * threadIdx.x + 3] = w[1];
+    // the same bytes straight to bf16 with the scale 2^9 that makes nibble n the number n
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+    const int packed = (int)(n | (n << 8) | (n << 16) | (n << 24));
+    const bf16x2 lo = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(packed, 512.0f, false);
+    const bf16x2 hi = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(packed, 512.0f, true);
+    out[64 + 4 * threadIdx.x] = (float)lo[0];
+    out[64 + 4 * threadIdx.x + 1] = (float)lo[1];
+    out[64 + 4 * threadIdx.x + 2] = (float)hi[0];
+    out[64 + 4 * threadIdx.x + 3] = (float)hi[1];
 }
 
 hipError_t probe_fp8_nibble_unit(hipStream_t stream, float *unit_out) {
     *unit_out = 0.f;
     float *d = nullptr;
-    hipError_t e = hipMalloc(reinterpret_cast<void **>(&d), 64 * sizeof(float));
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&d), 128 * sizeof(float));
     if (e != hipSuccess) return e;
-    float h[64];
+    float h[128];
     hipLaunchKernelGGL(fp8_nibble_probe, dim3(1), dim3(16), 0, stream, d);
     e = hipGetLastError();
     if (e == hipSuccess) e = hipMemcpyAsync(h, d, sizeof h, hipMemcpyDeviceToHost, stream);
@@ -2028,6 +2064,10 @@ hipError_t probe_fp8_nibble_unit(hipStream_t stream, float *unit_out) {
     int ex;
     if (linear && std::frexp(unit, &ex) != 0.5f) linear = false;
     *unit_out = linear ? unit : 0.f;
+    bool exact = true;  // fp8 -> bf16 with scale 512 must give the integers 0..15
+    for (int n = 0; n < 16; n++)
+        for (int k = 0; k < 4; k++) exact = exact && h[64 + 4 * n + k] == (float)n;
+    g_nibble_bf16 = exact;
     return hipSuccess;
 }
 
@@ -2262,6 +2302,7 @@ static bool mm_type(uint32_t type) { return type != T_F32 && type != T_F16 && ty
 struct MmPlan {
     MmBatch b;
     int tt;             // token tiles of 32 per workgroup (1 or 2)
+    uint32_t max_tok;   // most tokens of any job
     uint32_t n_groups;  // groups of 16 columns
     size_t xb_bytes, sx_bytes, part_bytes;
 };
@@ -2275,10 +2316,20 @@ static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *co
     uint32_t max_tok = 0, total_tok = 0;
     for (uint32_t j = 0; j < n; j++) max_tok = tokens[j] > max_tok ? tokens[j] : max_tok;
     p.tt = max_tok > 32 ? 2 : 1;
+    p.max_tok = max_tok;
     const uint32_t tile_tok = 32u * (uint32_t)p.tt;
     uint32_t wgs = 0;
     bool any_split = false;
     const uint32_t n_steps = mats[0].cols / 32;
+    // Columns are shared between workgroups only as far as the row and token tiles of the whole
+    // launch leave CUs idle: every share costs a partial result written and read back.
+    uint32_t launch_tiles = 0;
+    for (uint32_t j = 0; j < n; j++)
+        launch_tiles += ((tokens[j] + tile_tok - 1) / tile_tok) * ((mats[j].rows + MM_ROWS - 1) / MM_ROWS);
+    uint32_t ks_launch = (uint32_t)(2 * g_cu_count) / (launch_tiles ? launch_tiles : 1);  // two workgroups per CU (measured best of 1..4)
+    if (ks_launch > n_steps / 8) ks_launch = n_steps / 8;                                 // shares are whole 256-column units
+    if (ks_launch > 32) ks_launch = 32;
+    if (ks_launch < 1) ks_launch = 1;
     for (uint32_t j = 0; j < n; j++) {
         MmJob &job = b.job[j];
         job.m = mats[j];
@@ -2289,13 +2340,8 @@ static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *co
         job.tok_off = total_tok;
         job.wg_begin = wgs;
         job.tok_tiles = (tokens[j] + tile_tok - 1) / tile_tok;
-        // The column split of a product depends on that product alone, so that its
-        // result does not change with what else shares the launch.
         const uint32_t tiles = job.tok_tiles * ((mats[j].rows + MM_ROWS - 1) / MM_ROWS);
-        uint32_t ks = (uint32_t)(2 * g_cu_count) / tiles;  // two workgroups per CU (measured best of 1..4)
-        if (ks > n_steps / 8) ks = n_steps / 8;            // shares are whole 256-column units
-        if (ks > 32) ks = 32;
-        if (ks < 1) ks = 1;
+        uint32_t ks = ks_launch;
         job.ksplit = ks;
         job.pad = 0;
         wgs += tiles * ks;
@@ -2307,6 +2353,8 @@ static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *co
     b.mpad = total_tok + 64;  // a tile may read up to 63 slots past its job's last token
     b.total_wgs = wgs;
     b.any_split = any_split ? 1u : 0u;
+    b.nibble_bf16 = g_nibble_bf16 ? 1u : 0u;
+    b.pad0 = b.pad1 = b.pad2 = 0;
     p.n_groups = mats[0].cols / 16;
     p.xb_bytes = up256((size_t)p.n_groups * 6 * b.mpad * sizeof(uint4));
     p.sx_bytes = up256((size_t)p.n_groups * b.mpad * sizeof(float));
@@ -2316,9 +2364,13 @@ static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *co
     p.part_bytes = part;
 }
 
-template <uint32_t T, int TT> static hipError_t launch_mm_main(hipStream_t stream, const MmBatch &b) {
+template <uint32_t T, int TT, int VQ, bool FB = false>
+static hipError_t launch_mm_main(hipStream_t stream, const MmBatch &b) {
+    if constexpr (T == T_Q4_K && !FB) {
+        if (b.nibble_bf16) return launch_mm_main<T, TT, VQ, true>(stream, b);
+    }
     constexpr size_t lds = 2 * MmStage<T, TT>::BYTES;  // two pipeline stages
-    auto kern = gemm_mfma_kernel<T, TT>;
+    auto kern = gemm_mfma_kernel<T, TT, VQ, FB>;
     static bool configured = false;
     if (lds > 48 * 1024 && !configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -2346,7 +2398,12 @@ static hipError_t launch_mm_t(hipStream_t stream, MmPlan &p, void *ws, size_t ws
     const size_t split_threads = (size_t)p.n_groups * b.mpad;
     hipLaunchKernelGGL(mm_xsplit_kernel<T>, dim3((unsigned)((split_threads + 255) / 256)), dim3(256), 0, stream, b,
                        p.n_groups);
-    hipError_t e = p.tt == 1 ? launch_mm_main<T, 1>(stream, b) : launch_mm_main<T, 2>(stream, b);
+    hipError_t e;
+    if (p.tt == 2) e = launch_mm_main<T, 2, 4>(stream, b);
+    else if (p.max_tok <= 8) e = launch_mm_main<T, 1, 1>(stream, b);
+    else if (p.max_tok <= 16) e = launch_mm_main<T, 1, 2>(stream, b);
+    else if (p.max_tok <= 24) e = launch_mm_main<T, 1, 3>(stream, b);
+    else e = launch_mm_main<T, 1, 4>(stream, b);
     if (e != hipSuccess) return e;
     if (b.any_split) hipLaunchKernelGGL(mm_reduce_kernel, dim3(512, b.n_jobs), dim3(256), 0, stream, b);
     return hipGetLastError();

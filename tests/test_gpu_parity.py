@@ -344,14 +344,21 @@ def test_config5_expert_grouped_gemm(pkg, gpu):
             check(np.ascontiguousarray(ye[:, sample]), K.Q4_K, cols, tokens[e], sample.size, ws,
                   xs[buckets[e]].reshape(-1), f"config 5 expert {e}")
             assert np.all(np.isfinite(ye))
-        # one grouped call == the reference's sequence of per-expert calls
+        # one grouped call against the reference's sequence of per-expert calls: the same
+        # products, but a launch shares out columns by its total size, so the f32 sums may
+        # be formed in a different order
         y_seq = np.full_like(y, np.nan)
         yo = 0
         for e in range(n_exp):
             n = tokens[e] * rows
             gpu.gemm_resident(mats[e], tokens[e], xs[buckets[e]].reshape(-1), y_seq[yo:yo + n])
             yo += n
-        assert np.array_equal(y, y_seq)
+        rms = float(np.sqrt(np.mean(y_seq.astype(np.float64) ** 2)))
+        assert np.max(np.abs(y.astype(np.float64) - y_seq)) <= 2e-5 * rms
+        # and a repeated call is bit-identical (fixed summation order)
+        y_again = np.full_like(y, np.nan)
+        gpu.gemm_grouped(mats, tokens, x_packed, y_again)
+        assert np.array_equal(y, y_again)
         for mm in mats:
             mm.close()
 
