@@ -78,7 +78,10 @@ int lnh_upload_f32(lnh_exec *exec, size_t rows, size_t cols, const float *weight
  * the file and keeps them packed in HBM.  Replaces the host-side expansion to
  * F32 at langtax/src/quant.rs:6746-6755 followed by upload (native_gpu.rs:190-194).
  * `nbytes` must equal rows * row_bytes(type, cols); cols must be a whole number
- * of blocks (32 for Q4_0/Q5_0/Q5_1/Q8_0, 256 for Q4_K/Q6_K). */
+ * of blocks (32 for Q4_0/Q5_0/Q5_1/Q8_0, 256 for Q4_K/Q6_K).
+ * A quantized matrix is kept twice, in two layouts: one the single-token
+ * kernels stream, one the multi-token (matrix-core) kernels stream, so it takes
+ * about twice its GGUF size in HBM (lnh_matrix_info reports the exact figure). */
 int lnh_upload_packed(lnh_exec *exec, uint32_t ggml_type, size_t rows, size_t cols, const uint8_t *bytes,
                       size_t nbytes, lnh_matrix **out);
 /* Same, from bytes that already sit in device memory of this executor's GPU. */
@@ -113,7 +116,12 @@ int lnh_gemm_grouped(lnh_exec *exec, size_t n_groups, const lnh_matrix *const *m
 /* The same products with x and y already in this GPU's memory, enqueued on
  * `stream` (a hipStream_t; NULL = the executor's own stream) without any host
  * synchronisation.  No counterpart in the reference, whose every call copies
- * through the host (native-cuda/src/gpu.rs:301-303, 332-334). */
+ * through the host (native-cuda/src/gpu.rs:301-303, 332-334).
+ * Products of two or more tokens by a quantized matrix use a workspace that
+ * belongs to the executor and grows on demand (growing allocates, so it cannot
+ * happen while `stream` is being captured into a graph: run the largest shape
+ * once before capturing).  Calls of one executor must therefore be enqueued on
+ * one stream at a time; calls that overlap on different streams race on it. */
 int lnh_gemm_device(lnh_exec *exec, const lnh_matrix *matrix, size_t tokens, const float *device_x,
                     float *device_y, void *stream);
 int lnh_gemm_grouped_device(lnh_exec *exec, size_t n_groups, const lnh_matrix *const *mats,
