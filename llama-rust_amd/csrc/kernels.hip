@@ -40,6 +40,45 @@ __device__ __forceinline__ float dot4_ub(uint32_t q, const float *x, float acc) 
     return acc;
 }
 
+// Same with a code bias taken off every code before the multiply.  (Factoring the bias out
+// through the sum of x, sum q x - bias sum x, is cheaper but lets one large activation
+// under a zero weight swamp the small terms of the row: the two big numbers only
+// cancel at the end, after the accumulator has lost the small ones.)
+__device__ __forceinline__ float dot4_ub_biased(uint32_t q, float bias, const float *x, float acc) {
+    acc = fmaf(ub0(q) - bias, x[0], acc);
+    acc = fmaf(ub1(q) - bias, x[1], acc);
+    acc = fmaf(ub2(q) - bias, x[2], acc);
+    acc = fmaf(ub3(q) - bias, x[3], acc);
+    return acc;
+}
+// four signed bytes times four activations
+__device__ __forceinline__ float dot4_sb(uint32_t q, const float *x, float acc) {
+    acc = fmaf(sb(q, 0), x[0], acc);
+    acc = fmaf(sb(q, 1), x[1], acc);
+    acc = fmaf(sb(q, 2), x[2], acc);
+    acc = fmaf(sb(q, 3), x[3], acc);
+    return acc;
+}
+// Low nibble of byte K of w, read as a signed 4-bit integer, divided by 16 (v_cvt_off_f32_i4 with a
+// byte select, so that no shift is spent on picking the byte).  With w = codes ^ 0x88888888 that
+// is (n - 8) / 16 for the nibble n.
+template <int K> __device__ __forceinline__ float i4_of_byte(uint32_t w) {
+    float r;
+    if constexpr (K == 0) asm("v_cvt_off_f32_i4_sdwa %0, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(r) : "v"(w));
+    if constexpr (K == 1) asm("v_cvt_off_f32_i4_sdwa %0, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1" : "=v"(r) : "v"(w));
+    if constexpr (K == 2) asm("v_cvt_off_f32_i4_sdwa %0, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(r) : "v"(w));
+    if constexpr (K == 3) asm("v_cvt_off_f32_i4_sdwa %0, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3" : "=v"(r) : "v"(w));
+    return r;
+}
+// sum over the low nibbles of the four bytes of w (signed, / 16) times four activations
+__device__ __forceinline__ float dot4_i4(uint32_t w, const float *x, float acc) {
+    acc = fmaf(i4_of_byte<0>(w), x[0], acc);
+    acc = fmaf(i4_of_byte<1>(w), x[1], acc);
+    acc = fmaf(i4_of_byte<2>(w), x[2], acc);
+    acc = fmaf(i4_of_byte<3>(w), x[3], acc);
+    return acc;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
@@ -381,6 +420,14 @@ __device__ __forceinline__ uint32_t q5_bytes(uint32_t nib, uint32_t qh, int e0) 
     return nib | (spread << 4);
 }
 
+// Same for Q5_0 as signed bytes 8 (c - 16): nib8 holds the nibbles in bits 3..6 of every byte, the
+// fifth bit goes to bit 7 and is flipped (c ^ 16 is c - 16 in 5-bit two's complement).
+__device__ __forceinline__ uint32_t q5_signed_bytes(uint32_t nib8, uint32_t qh, int e0) {
+    uint32_t h4 = (qh >> e0) & 0xfu;
+    uint32_t spread = (h4 * 0x00204081u) & 0x01010101u;
+    return (nib8 | (spread << 7)) ^ 0x80808080u;
+}
+
 // Contribution of one chunk of one row to that row's dot product.
 template <uint32_t T>
 __device__ __forceinline__ float chunk_dot(const Raw<T> &r, const XChunk<Geo<T>::E> &xc, uint32_t c, float acc) {
@@ -413,22 +460,20 @@ __device__ __forceinline__ float chunk_dot(const Raw<T> &r, const XChunk<Geo<T>:
         float t = 0.f;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            t = dot4_ub(w[i] & 0x0f0f0f0fu, x + 4 * i, t);
-            t = dot4_ub((w[i] >> 4) & 0x0f0f0f0fu, x + 16 + 4 * i, t);
+            t = dot4_ub_biased(w[i] & 0x0f0f0f0fu, 8.f, x + 4 * i, t);
+            t = dot4_ub_biased((w[i] >> 4) & 0x0f0f0f0fu, 8.f, x + 16 + 4 * i, t);
         }
-        // sum (n - 8) x = sum n x - 8 sum x
-        t = fmaf(-8.f, xc.s_lo + xc.s_hi, t);
         return fmaf(h2f(r.d), t, acc);
     } else if constexpr (T == T_Q5_0 || T == T_Q5_1) {
         const uint32_t w[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
         float t = 0.f;
+        constexpr float bias = T == T_Q5_0 ? 16.f : 0.f;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            t = dot4_ub(q5_bytes(w[i] & 0x0f0f0f0fu, r.qh, 4 * i), x + 4 * i, t);
-            t = dot4_ub(q5_bytes((w[i] >> 4) & 0x0f0f0f0fu, r.qh, 16 + 4 * i), x + 16 + 4 * i, t);
+            t = dot4_ub_biased(q5_bytes(w[i] & 0x0f0f0f0fu, r.qh, 4 * i), bias, x + 4 * i, t);
+            t = dot4_ub_biased(q5_bytes((w[i] >> 4) & 0x0f0f0f0fu, r.qh, 16 + 4 * i), bias, x + 16 + 4 * i, t);
         }
         if constexpr (T == T_Q5_0) {
-            t = fmaf(-16.f, xc.s_lo + xc.s_hi, t);
             return fmaf(h2f(r.d), t, acc);
         } else {
             float d = h2f((uint16_t)(r.dm & 0xffffu)), mm = h2f((uint16_t)(r.dm >> 16));
@@ -463,12 +508,9 @@ __device__ __forceinline__ float chunk_dot(const Raw<T> &r, const XChunk<Geo<T>:
         for (int i = 0; i < 4; i++) {
             uint32_t two_lo = (hb[i] >> (2 * h)) & 0x03030303u;        // quarter h
             uint32_t two_hi = (hb[i] >> (2 * h + 4)) & 0x03030303u;    // quarter h + 2
-            tl = dot4_ub((lo[i] & 0x0f0f0f0fu) | (two_lo << 4), x + 4 * i, tl);
-            th = dot4_ub(((lo[i] >> 4) & 0x0f0f0f0fu) | (two_hi << 4), x + 16 + 4 * i, th);
+            tl = dot4_ub_biased((lo[i] & 0x0f0f0f0fu) | (two_lo << 4), 32.f, x + 4 * i, tl);
+            th = dot4_ub_biased(((lo[i] >> 4) & 0x0f0f0f0fu) | (two_hi << 4), 32.f, x + 16 + 4 * i, th);
         }
-        // codes are biased by 32: sum (q - 32) x = sum q x - 32 sum x
-        tl = fmaf(-32.f, xc.s_lo, tl);
-        th = fmaf(-32.f, xc.s_hi, th);
         int sh = 8 * (2 * h + k);
         float s_lo = (float)(int)(int8_t)(r.sc.x >> sh);  // scale 8n + 2h + k
         float s_hi = (float)(int)(int8_t)(r.sc.y >> sh);  // scale 8n + 2(h+2) + k
@@ -892,9 +934,9 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b,
 // Piece cc of ql (n = cc>>2, p = (cc>>1)&1, lh = cc&1) holds in its low nibbles 16
 // codes of quarter p and in its high nibbles 16 codes of quarter p+2 of half n; their
 // two high bits sit in qh piece 2n+lh at bit 2p resp. 2p+4 (langtax/src/quant.rs:8783-8853).
-// The 6-bit codes are assembled four to a register and converted with v_cvt_f32_ubyte;
-// the bias of 32 and the sixteen int8 scales are applied per 16 columns through
-// sum_s sc_s * (sum_k q_k x_k - 32 sum_k x_k).
+// The 6-bit codes are assembled four to a register, converted with v_cvt_f32_ubyte and
+// brought back to -32..31 before the multiply; the sixteen int8 scales are applied per
+// 16 columns.
 
 struct Q6kUnit {
     uint4 ql[8], qh[4], sc;
@@ -912,7 +954,6 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q6k_kernel(const GemvBatch b)
     const float *xw = b.x + (size_t)b.unit0 * 256;
     const uint32_t n_iter = (nb + LB - 1) / LB;
     float *xs = lds;                                  // as in the Q4_K kernel, with this dtype's column order
-    float *ssum = lds + (size_t)n_iter * XS_FLOATS;   // [it][16 column groups][blk % LB]
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -959,10 +1000,6 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q6k_kernel(const GemvBatch b)
         const uint32_t cc = 4 * n + 2 * (quarter & 1u) + (l >> 4), t = (quarter >> 1) * 16 + (l & 15u);
         const uint32_t it = blk / LB, bl = blk % LB;
         *reinterpret_cast<float4 *>(xs + (size_t)it * XS_FLOATS + (cc * 8 + (t >> 2)) * XROW + bl * 4) = v;
-        float sm = (v.x + v.y) + (v.z + v.w);
-        sm += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0xb1, 0xf, 0xf, false));
-        sm += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0x4e, 0xf, 0xf, false));
-        if ((lane & 3u) == 0) ssum[(it * 16 + (r >> 4)) * LB + bl] = sm;
     };
     for (uint32_t col = tid * 4; col < n_iter * LB * 256; col += NW * 64 * 4)
         stage(col, *reinterpret_cast<const float4 *>(xw + (col < cols ? col : 0)));
@@ -995,15 +1032,16 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q6k_kernel(const GemvBatch b)
             float tl = 0.f, th = 0.f;
 #pragma unroll
             for (int d = 0; d < 4; d++) {
-                const uint32_t two_lo = p == 0 ? (hb[d] << 4) : (hb[d] << 2);   // bits 2p..2p+1 moved to 4..5
-                const uint32_t two_hi = p == 0 ? hb[d] : (hb[d] >> 2);          // bits 2p+4..2p+5 moved to 4..5
-                tl = dot4_ub((lo[d] & 0x0f0f0f0fu) | (two_lo & 0x30303030u), x + 4 * d, tl);
-                th = dot4_ub(((lo[d] >> 4) & 0x0f0f0f0fu) | (two_hi & 0x30303030u), x + 16 + 4 * d, th);
+                // Each byte becomes 4 (q - 32) as a signed byte: the 6-bit code in bits 2..7 with its top
+                // bit flipped (q ^ 32 is q - 32 in 6-bit two's complement).  The 4 goes into the scale.
+                const uint32_t two_lo = p == 0 ? (hb[d] << 6) : (hb[d] << 4);   // bits 2p..2p+1 moved to 6..7
+                const uint32_t two_hi = p == 0 ? (hb[d] << 2) : hb[d];          // bits 2p+4..2p+5 moved to 6..7
+                tl = dot4_sb((((lo[d] << 2) & 0x3c3c3c3cu) | (two_lo & 0xc0c0c0c0u)) ^ 0x80808080u, x + 4 * d, tl);
+                th = dot4_sb((((lo[d] >> 2) & 0x3c3c3c3cu) | (two_hi & 0xc0c0c0c0u)) ^ 0x80808080u, x + 16 + 4 * d, th);
             }
             t[8 * n + 2 * p + lh] = tl;        // scale index 8n + lh + 2*quarter, quarter = p
             t[8 * n + 2 * (p + 2) + lh] = th;  // quarter = p + 2
         }
-        const float *sp = ssum + (size_t)it * 16 * LB + b0;
         const uint32_t scw[4] = {un.sc.x, un.sc.y, un.sc.z, un.sc.w};
         float S = 0.f;
 #pragma unroll
@@ -1011,9 +1049,9 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q6k_kernel(const GemvBatch b)
             // t index k = 8n + 2*quarter + lh is also the int8 scale index; the matching 16-column
             // group of x is (8n + 2*quarter + lh) in column order: group = r >> 4 with r = 128n + 32q + 16lh
             const float sc = (float)(int)(int8_t)(scw[k >> 2] >> (8 * (k & 3)));
-            S = fmaf(sc, fmaf(-32.f, sp[k * LB], t[k]), S);
+            S = fmaf(sc, t[k], S);
         }
-        const float part = h2f(un.d) * S;
+        const float part = (h2f(un.d) * 0.25f) * S;  // t holds 4 (q - 32) sums
         acc += active ? part : 0.f;
         if (it + 1 == n_iter) {
             const Where w = locate(g);
@@ -1032,8 +1070,9 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q6k_kernel(const GemvBatch b)
 // 4 blocks (128 columns) of Q8_0, i.e. 8 code pieces of 16 bytes (piece-major, see
 // matview.h) plus the unit's scales, which are contiguous in their plane.  x sits in
 // LDS in column order, one float4 row per 4 columns of a unit, padded like the
-// Q4_K kernel's.  Code biases (8, 16, 128) and Q5_1's offsets go through the
-// per-block sums of x:  sum_k d (q_k - bias) x_k = d (sum_k q_k x_k - bias sum_k x_k)
+// Q4_K kernel's.  Codes are brought to their signed value before the multiply
+// (Q8_0: signed byte convert; Q4_0: signed 4-bit convert; Q5_0: minus 16); only Q5_1's
+// offsets, which are separate terms of the weight, go through the per-block sums of x
 // (langtax/src/quant.rs:7511-7541, 7734-7765, 7884-7950, 8046-8130).
 
 template <uint32_t T> struct B32Geo {
@@ -1047,8 +1086,9 @@ template <> struct B32Unit<T_Q4_0> { uint4 q[8]; uint4 d; };
 template <> struct B32Unit<T_Q5_0> { uint4 q[8]; uint4 qh[2]; uint4 d; };
 template <> struct B32Unit<T_Q5_1> { uint4 q[8]; uint4 qh[2]; uint4 dm[2]; };
 
-template <uint32_t T, int LB, int NW, bool FP8>
-__global__ __launch_bounds__(NW * 64, (T == T_Q5_0 || T == T_Q5_1) ? 3 : 4) void gemv_b32_kernel(const GemvBatch b, const float nib_mul, const float nib_unit) {
+// I4: Q4_0 nibbles go through the signed 4-bit convert (else byte convert and subtract).
+template <uint32_t T, int LB, int NW, bool I4>
+__global__ __launch_bounds__(NW * 64, (T == T_Q5_0 || T == T_Q5_1) ? 3 : 4) void gemv_b32_kernel(const GemvBatch b) {
     using G = B32Geo<T>;
     constexpr uint32_t RS = 64 / LB;           // rows per wavefront step = rows per row group
     constexpr uint32_t XROW = LB * 4 + 4;      // floats per LDS row: LB float4 plus one of padding
@@ -1129,13 +1169,15 @@ __global__ __launch_bounds__(NW * 64, (T == T_Q5_0 || T == T_Q5_1) ? 3 : 4) void
     auto stage = [&](uint32_t col, const float4 v) {
         const uint32_t un = col / G::UC, e = col % G::UC, it = un / LB, bl = un % LB;
         *reinterpret_cast<float4 *>(xs + (size_t)it * XS_FLOATS + (e >> 2) * XROW + bl * 4) = v;
-        float sm = (v.x + v.y) + (v.z + v.w);
+        if constexpr (T == T_Q5_1) {  // the offsets m multiply the block sums of x
+            float sm = (v.x + v.y) + (v.z + v.w);
 #define NH_DPP_ADD(ctrl) sm += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), ctrl, 0xf, 0xf, false))
-        NH_DPP_ADD(0xb1);
-        NH_DPP_ADD(0x4e);
-        NH_DPP_ADD(0x141);
+            NH_DPP_ADD(0xb1);
+            NH_DPP_ADD(0x4e);
+            NH_DPP_ADD(0x141);
 #undef NH_DPP_ADD
-        if ((lane & 7u) == 0) ssum[(it * G::NBLK + (e >> 5)) * LB + bl] = sm;
+            if ((lane & 7u) == 0) ssum[(it * G::NBLK + (e >> 5)) * LB + bl] = sm;
+        }
     };
     constexpr int NXV = (LB * G::UC / 4 + NW * 64 - 1) / (NW * 64);  // float4 per thread for LB units of x
     if (n_iter == 1) {
@@ -1187,11 +1229,20 @@ __global__ __launch_bounds__(NW * 64, (T == T_Q5_0 || T == T_Q5_1) ? 3 : 4) void
 #pragma unroll
             for (int d = 0; d < 4; d++) {
                 if constexpr (T == T_Q8_0) {
-                    // signed byte + 128 as an unsigned byte; the 128 comes back out through the sum of x
-                    t[cc >> 1] = dot4_ub(w[d] ^ 0x80808080u, x + 4 * d, t[cc >> 1]);
+                    t[cc >> 1] = dot4_sb(w[d], x + 4 * d, t[cc >> 1]);
                 } else if constexpr (T == T_Q4_0) {
-                    t[cc] = dot4_nib<FP8>(w[d] & 0x0f0f0f0fu, x + 4 * d, t[cc]);
-                    t[cc] = dot4_nib<FP8>((w[d] >> 4) & 0x0f0f0f0fu, x + 16 + 4 * d, t[cc]);
+                    if constexpr (I4) {  // (n - 8) / 16 per nibble; the 16 goes into the block scale
+                        const uint32_t wx = w[d] ^ 0x88888888u;
+                        t[cc] = dot4_i4(wx, x + 4 * d, t[cc]);
+                        t[cc] = dot4_i4(wx >> 4, x + 16 + 4 * d, t[cc]);
+                    } else {
+                        t[cc] = dot4_ub_biased(w[d] & 0x0f0f0f0fu, 8.f, x + 4 * d, t[cc]);
+                        t[cc] = dot4_ub_biased((w[d] >> 4) & 0x0f0f0f0fu, 8.f, x + 16 + 4 * d, t[cc]);
+                    }
+                } else if constexpr (T == T_Q5_0) {
+                    // bytes 8 (c - 16): the 5-bit code in bits 3..7 with its top bit flipped; the 8 goes into the scale
+                    t[cc] = dot4_sb(q5_signed_bytes((w[d] << 3) & 0x78787878u, qh[cc], 4 * d), x + 4 * d, t[cc]);
+                    t[cc] = dot4_sb(q5_signed_bytes((w[d] >> 1) & 0x78787878u, qh[cc], 16 + 4 * d), x + 16 + 4 * d, t[cc]);
                 } else {
                     t[cc] = dot4_ub(q5_bytes(w[d] & 0x0f0f0f0fu, qh[cc], 4 * d), x + 4 * d, t[cc]);
                     t[cc] = dot4_ub(q5_bytes((w[d] >> 4) & 0x0f0f0f0fu, qh[cc], 16 + 4 * d), x + 16 + 4 * d, t[cc]);
@@ -1204,17 +1255,14 @@ __global__ __launch_bounds__(NW * 64, (T == T_Q5_0 || T == T_Q5_1) ? 3 : 4) void
 #pragma unroll
             for (int k = 0; k < 4; k++) {
                 const float d = h2f((uint16_t)(dd[k >> 1] >> (16 * (k & 1))));
-                part = fmaf(d, fmaf(-128.f, sp[k * LB], t[k]), part);
+                part = fmaf(d, t[k], part);
             }
         } else if constexpr (T == T_Q4_0 || T == T_Q5_0) {
             const uint32_t dd[4] = {q.d.x, q.d.y, q.d.z, q.d.w};
 #pragma unroll
             for (int k = 0; k < 8; k++) {
                 const float d = h2f((uint16_t)(dd[k >> 1] >> (16 * (k & 1))));
-                if constexpr (T == T_Q4_0)  // t holds nib_unit * sum n x when the fp8 unpack is in use
-                    part = fmaf(d * nib_mul, fmaf(-8.f * nib_unit, sp[k * LB], t[k]), part);
-                else
-                    part = fmaf(d, fmaf(-16.f, sp[k * LB], t[k]), part);
+                part = fmaf(T == T_Q5_0 ? d * 0.125f : (I4 ? d * 16.f : d), t[k], part);
             }
         } else {
             const uint32_t dm[8] = {q.dm[0].x, q.dm[0].y, q.dm[0].z, q.dm[0].w, q.dm[1].x, q.dm[1].y, q.dm[1].z, q.dm[1].w};
@@ -1732,10 +1780,8 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const MmBatch b) {
     static_assert(XR <= 3, "XbRegs holds three vectors");
     float sx0 = 0.f, sx1 = 0.f, sx2 = 0.f, sx3 = 0.f;
 
-    // Offsets are applied once per 32 columns that share them: Q5_1 every step
-    // (one block), Q4_K on even steps (a sub-block spans the same group of two
-    // consecutive steps).
-    auto offset_step = [](uint32_t s) { return T == T_Q5_1 || (s & 1u) == 0; };
+    // Offsets are applied once per 32 columns that share them: Q5_1 every step (one block),
+    // Q4_K on even steps (a sub-block spans the same group of two consecutive steps).
 
     // Every fetch issues the same loads whatever the step and the thread (indices
     // are clamped instead of branching), so that the number of loads in flight is
@@ -1973,6 +2019,7 @@ __global__ __launch_bounds__(256) void mm_reduce_kernel(const MmBatch b) {
 // ------------------------------------------------------------------ launchers
 
 static bool g_nibble_bf16 = false;  // the packed fp8 -> bf16 convert turns nibble bytes into the integers 0..15
+static bool g_nibble_i4 = false;    // the signed 4-bit convert with a byte select gives (n - 8) / 16 for nibble n ^ 8
 static int g_cu_count = 256;
 static size_t g_lds_limit = 64 * 1024;
 
@@ -2042,14 +2089,24 @@ __global__ void fp8_nibble_probe(float *out) {
     out[64 + 4 * threadIdx.x + 1] = (float)lo[1];
     out[64 + 4 * threadIdx.x + 2] = (float)hi[0];
     out[64 + 4 * threadIdx.x + 3] = (float)hi[1];
+    // signed 4-bit convert of the low nibble of every byte, and of the high nibbles after a shift
+    const uint32_t lo_n = (n | (n << 8) | (n << 16) | (n << 24)) ^ 0x88888888u, hi_n = ((n << 4) * 0x01010101u) ^ 0x88888888u;
+    out[128 + 8 * threadIdx.x] = i4_of_byte<0>(lo_n);
+    out[128 + 8 * threadIdx.x + 1] = i4_of_byte<1>(lo_n);
+    out[128 + 8 * threadIdx.x + 2] = i4_of_byte<2>(lo_n);
+    out[128 + 8 * threadIdx.x + 3] = i4_of_byte<3>(lo_n);
+    out[128 + 8 * threadIdx.x + 4] = i4_of_byte<0>(hi_n >> 4);
+    out[128 + 8 * threadIdx.x + 5] = i4_of_byte<1>(hi_n >> 4);
+    out[128 + 8 * threadIdx.x + 6] = i4_of_byte<2>(hi_n >> 4);
+    out[128 + 8 * threadIdx.x + 7] = i4_of_byte<3>(hi_n >> 4);
 }
 
 hipError_t probe_fp8_nibble_unit(hipStream_t stream, float *unit_out) {
     *unit_out = 0.f;
     float *d = nullptr;
-    hipError_t e = hipMalloc(reinterpret_cast<void **>(&d), 128 * sizeof(float));
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&d), 256 * sizeof(float));
     if (e != hipSuccess) return e;
-    float h[128];
+    float h[256];
     hipLaunchKernelGGL(fp8_nibble_probe, dim3(1), dim3(16), 0, stream, d);
     e = hipGetLastError();
     if (e == hipSuccess) e = hipMemcpyAsync(h, d, sizeof h, hipMemcpyDeviceToHost, stream);
@@ -2068,6 +2125,10 @@ hipError_t probe_fp8_nibble_unit(hipStream_t stream, float *unit_out) {
     for (int n = 0; n < 16; n++)
         for (int k = 0; k < 4; k++) exact = exact && h[64 + 4 * n + k] == (float)n;
     g_nibble_bf16 = exact;
+    exact = true;
+    for (int n = 0; n < 16; n++)
+        for (int k = 0; k < 8; k++) exact = exact && h[128 + 8 * n + k] == (float)(n - 8) / 16.0f;
+    g_nibble_i4 = exact;
     return hipSuccess;
 }
 
@@ -2195,7 +2256,7 @@ static hipError_t launch_gemv_q6k(hipStream_t stream, const MatView *mats, float
         b.unit0 = win.first(w);
         b.units = units;
         b.accumulate = w > 0;
-        const size_t lds = (size_t)(64 * (lb * 4 + 4) + lb * 16) * sizeof(float);
+        const size_t lds = (size_t)(64 * (lb * 4 + 4)) * sizeof(float);
         if (lds > g_lds_limit) return hipErrorInvalidValue;
         hipError_t e;
         switch (lb) {
@@ -2214,7 +2275,7 @@ static hipError_t launch_gemv_q6k(hipStream_t stream, const MatView *mats, float
 
 template <uint32_t T, int LB, int NW>
 static hipError_t launch_b32_lb(hipStream_t stream, const GemvBatch &b, uint32_t units, size_t lds) {
-    const bool fp8 = T == T_Q4_0 && g_nib_mul != 0.f;
+    const bool fp8 = T == T_Q4_0 && g_nibble_i4;  // which of the two instantiations
     const void *kern = fp8 ? reinterpret_cast<const void *>(gemv_b32_kernel<T, LB, NW, true>)
                            : reinterpret_cast<const void *>(gemv_b32_kernel<T, LB, NW, false>);
     static size_t configured[2] = {0, 0};
@@ -2229,11 +2290,10 @@ static hipError_t launch_b32_lb(hipStream_t stream, const GemvBatch &b, uint32_t
     uint32_t grid = (uint32_t)((size_t)g_cu_count * per_cu);
     const uint32_t needed = (units + NW - 1) / NW;
     if (grid > needed) grid = needed;
-    const float mul = fp8 ? g_nib_mul : 1.0f, unit = fp8 ? 1.0f / g_nib_mul : 1.0f;
     if (fp8)
-        hipLaunchKernelGGL((gemv_b32_kernel<T, LB, NW, true>), dim3(grid), dim3(NW * 64), lds, stream, b, mul, unit);
+        hipLaunchKernelGGL((gemv_b32_kernel<T, LB, NW, true>), dim3(grid), dim3(NW * 64), lds, stream, b);
     else
-        hipLaunchKernelGGL((gemv_b32_kernel<T, LB, NW, false>), dim3(grid), dim3(NW * 64), lds, stream, b, mul, unit);
+        hipLaunchKernelGGL((gemv_b32_kernel<T, LB, NW, false>), dim3(grid), dim3(NW * 64), lds, stream, b);
     return hipGetLastError();
 }
 

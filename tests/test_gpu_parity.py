@@ -209,6 +209,52 @@ def test_random_gemv_and_gemm_within_bounds(pkg, gpu, ty):
 
 
 @pytest.mark.parametrize("ty", [K.Q4_0, K.Q5_0, K.Q5_1, K.Q8_0, K.Q4_K, K.Q6_K], ids=lambda t: O.TYPE_NAMES[t])
+def test_adversarial_activations_keep_the_reference_bound(pkg, gpu, ty):
+    """The multi-token kernels hand the f32 activations to the matrix cores as three bf16 numbers
+    each.  That is only a faithful f32 product (the reference never rounds activations,
+    langtax/src/quant.rs:6760-6888) if the three parts carry all 24 significand bits at every
+    magnitude: full-mantissa values, 2^-60 .. 2^60 in one row, signed zeros, tiny values."""
+    rng = np.random.default_rng(4242 + ty)
+    rows, cols, tokens = 96, 2048, 6
+    w = K.random_packed(ty, rows, cols, rng)
+    m = gpu.upload_packed(ty, rows, cols, w)
+    mant = rng.integers(0, 1 << 23, size=(tokens, cols)).astype(np.uint32)
+    sign = rng.integers(0, 2, size=(tokens, cols)).astype(np.uint32) << 31
+    x = np.empty((tokens, cols), np.float32)
+    # token 0: every significand bit set, exponent 0;  token 1: random full mantissas
+    x[0] = (np.uint32(0x3F800000) | np.uint32(0x7FFFFF) | sign[0]).view(np.float32)
+    x[1] = (np.uint32(0x3F800000) | mant[1] | sign[1]).view(np.float32)
+    # token 2: exponents spread over 2^-60 .. 2^60 within the row
+    e2 = rng.integers(127 - 60, 127 + 61, size=cols).astype(np.uint32) << 23
+    x[2] = (e2 | mant[2] | sign[2]).view(np.float32)
+    # token 3: tiny but normal values (2^-100), token 4: zeros of both signs among ordinary values
+    x[3] = ((np.uint32(27) << 23) | mant[3] | sign[3]).view(np.float32)
+    x[4] = rng.normal(0, 1, cols).astype(np.float32)
+    x[4, ::3] = 0.0
+    x[4, 1::3] = -0.0
+    # token 5: one large value among small ones (cancellation in the other columns must survive)
+    x[5] = rng.normal(0, 1e-3, cols).astype(np.float32)
+    x[5, 777] = 3.0e4
+    y = np.full(tokens * rows, np.nan, np.float32)
+    gpu.gemm_resident(m, tokens, x.reshape(-1), y)
+    exact, mag = O.gemm_f64_mag(ty, cols, tokens, w, x.reshape(-1), rows)
+    err = np.abs(y.reshape(tokens, rows).astype(np.float64) - exact)
+    assert np.all(np.isfinite(y))
+    # the reference's proven bound and its observed envelope, per output, relative to sum |w x|
+    assert np.all(err <= K.single_kernel_bound(cols, mag))
+    assert np.all(err <= K.observed_envelope_u(cols) * K.U * mag)
+    # the single-token kernels on the same rows: the same bounds (a code bias factored out
+    # through the sum of x would fail here: one large activation under a zero weight)
+    for t in range(tokens):
+        y1 = np.full(rows, np.nan, np.float32)
+        gpu.gemv_resident(m, x[t], y1)
+        err1 = np.abs(y1.astype(np.float64) - exact[t])
+        assert np.all(err1 <= K.single_kernel_bound(cols, mag[t])), f"token {t}"
+        assert np.all(err1 <= K.observed_envelope_u(cols) * K.U * mag[t]), f"token {t}"
+    m.close()
+
+
+@pytest.mark.parametrize("ty", [K.Q4_0, K.Q5_0, K.Q5_1, K.Q8_0, K.Q4_K, K.Q6_K], ids=lambda t: O.TYPE_NAMES[t])
 def test_every_f16_scale_pattern_and_zero_blocks(pkg, gpu, ty):
     """langtax/src/simd/tests.rs:795-828, 1481-1520: every finite binary16 pattern as a block
     scale (subnormals must survive the hardware conversion), and all-zero blocks."""
