@@ -1710,23 +1710,38 @@ __device__ __forceinline__ void mm_decode(const MmRaw<T> &raw, uint32_t s, uint4
     }
 }
 
-// LDS of one pipeline stage (one step of 32 columns for the workgroup's 256 rows).
+// LDS of one pipeline stage: the split activations of one step of 32 columns for the
+// workgroup's tokens (the weights never pass through LDS).
 template <uint32_t T, int TT> struct MmStage {
     static constexpr bool OFFSET = MmTraits<T>::OFFSET;
     static constexpr int TOK = 32 * TT;
-    static constexpr int XB_VEC = 12 * TOK;  // [group][part][half][token] x 16 bytes
-    static constexpr size_t CODE = 0;                                   // uint4 [2][2][256]
-    static constexpr size_t SCALE = CODE + (size_t)4 * MM_ROWS * 16;    // float [2][256]
-    static constexpr size_t OFFS = SCALE + (size_t)2 * MM_ROWS * 4;     // float [2][256]
-    static constexpr size_t XB = OFFS + (OFFSET ? (size_t)2 * MM_ROWS * 4 : 0);
+    static constexpr int XB_VEC = 12 * TOK;                             // [group][part][half][token] x 16 bytes
     static constexpr int XB_SLOTS = (XB_VEC + 255) / 256 * 256;        // every thread stores whole vectors, no tail branch
+    static constexpr size_t XB = 0;
     static constexpr size_t SX = XB + (size_t)XB_SLOTS * 16;            // float [2][TOK], padded to one per thread
     static constexpr size_t BYTES = SX + (OFFSET ? (size_t)256 * 4 : 0);
 };
 
+// Lanes l and l + 32 exchange: a[l + 32] <-> b[l] (v_permlane32_swap).  Afterwards a holds, in
+// both halves of the wavefront, what the lower half had (a's old lower half, b's old lower
+// half) and b what the upper half had.
+__device__ __forceinline__ void swap32(uint32_t &a, uint32_t &b) {
+    const auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+    a = r[0];
+    b = r[1];
+}
+
 // TT: token tiles of 32 per workgroup.  VQ: how many of a tile's four 8-token quads can hold
 // tokens (a lane's accumulator v belongs to quad v / 4); the others are neither scaled nor stored.
 // FB: nibble bytes go straight to bf16 with the packed fp8 convert (Q4_K, when the device probe allows).
+//
+// A wavefront owns 64 rows and decodes them itself, one row per lane: 16 codes per group as
+// two halves of 8 bf16.  The MFMA wants, for the 32 rows of a row set, the first halves in
+// lanes 0..31 and the second halves in lanes 32..63 - one v_permlane32_swap per register gives
+// exactly that for both row sets at once (lower half: rows 0..31's first halves and rows
+// 32..63's first halves; upper half: the second halves), so the weights never touch LDS and
+// no barrier stands between a wavefront's decode and its MFMAs.  Only the split activations,
+// which all four wavefronts read, go through LDS (two stages, one barrier per step).
 template <uint32_t T, int TT, int VQ, bool FB>
 __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const MmBatch b) {
     constexpr int NV = 4 * VQ;
@@ -1780,15 +1795,17 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const MmBatch b) {
     static_assert(XR <= 3, "XbRegs holds three vectors");
     float sx0 = 0.f, sx1 = 0.f, sx2 = 0.f, sx3 = 0.f;
 
-    // Offsets are applied once per 32 columns that share them: Q5_1 every step (one block),
-    // Q4_K on even steps (a sub-block spans the same group of two consecutive steps).
-
     // Every fetch issues the same loads whatever the step and the thread (indices
     // are clamped instead of branching), so that the number of loads in flight is
     // known at compile time and a wait for the oldest step does not wait for all.
-    auto fetch = [&](uint32_t s_want, MmRaw<T> &raw, XbRegs &xbr, float &sxr) {
+    auto fetch_w = [&](uint32_t s_want, MmRaw<T> &raw) {
         const uint32_t s = s_want < s_end ? s_want : s_end - 1;
         mm_load<T>(m, tile_r, tid, s, raw);
+    };
+    // Offsets are applied once per 32 columns that share them: Q5_1 every step (one block),
+    // Q4_K on even steps (a sub-block spans the same group of two consecutive steps).
+    auto fetch_x = [&](uint32_t s_want, XbRegs &xbr, float &sxr) {
+        const uint32_t s = s_want < s_end ? s_want : s_end - 1;
         const uint4 *src = b.xb + (size_t)s * 12 * mpad + slot0;
 #pragma unroll
         for (int r = 0; r < XR; r++) {
@@ -1807,52 +1824,50 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const MmBatch b) {
             sxr = b.sx[g0 * mpad + slot0 + i] + b.sx[g1 * mpad + slot0 + i];
         }
     };
-    auto store = [&](uint32_t s_want, uint32_t buf, const MmRaw<T> &raw, const XbRegs &xbr, const float &sxr) {
-        const uint32_t s = s_want < s_end ? s_want : s_end - 1;  // past the end: decodes the clamped fetch, never read
+    auto stage_x = [&](uint32_t buf, const XbRegs &xbr, const float &sxr) {
         uint8_t *st = mm_lds + (size_t)buf * St::BYTES;
-        uint4 frag[2][2];
-        float sc[2], of[2];
-        mm_decode<T, FB>(raw, s, frag, sc, of);
-        uint4 *code_s = reinterpret_cast<uint4 *>(st + St::CODE);
-        float *scale_s = reinterpret_cast<float *>(st + St::SCALE);
-#pragma unroll
-        for (int g = 0; g < 2; g++) {
-            code_s[(2 * g) * MM_ROWS + tid] = frag[g][0];
-            code_s[(2 * g + 1) * MM_ROWS + tid] = frag[g][1];
-            scale_s[g * MM_ROWS + tid] = sc[g];
-            if constexpr (OFFSET) reinterpret_cast<float *>(st + St::OFFS)[g * MM_ROWS + tid] = of[g];
-        }
         uint4 *xb_s = reinterpret_cast<uint4 *>(st + St::XB);
 #pragma unroll
         for (int r = 0; r < XR; r++) {
             const uint32_t v = tid + 256 * r;
             xb_s[v] = r == 0 ? xbr.v0 : r == 1 ? xbr.v1 : xbr.v2;  // slots past XB_VEC are padding
         }
-        if constexpr (OFFSET) {
-            reinterpret_cast<float *>(st + St::SX)[tid] = sxr;  // read only on offset steps, entries [0, 2 TOK)
-        }
+        if constexpr (OFFSET) reinterpret_cast<float *>(st + St::SX)[tid] = sxr;  // read on offset steps, entries [0, 2 TOK)
     };
     // even_step: s is even (known at compile time: shares of K-quant rows start at a multiple of 8 steps)
-    auto compute = [&](uint32_t s, uint32_t buf, auto even_step) {
+    auto compute = [&](uint32_t s, uint32_t buf, const MmRaw<T> &raw, auto even_step) {
+        constexpr bool with_offset = OFFSET && (T == T_Q5_1 || decltype(even_step)::value);
         const uint8_t *st = mm_lds + (size_t)buf * St::BYTES;
-        const uint4 *code_s = reinterpret_cast<const uint4 *>(st + St::CODE);
-        const float *scale_s = reinterpret_cast<const float *>(st + St::SCALE);
-        const float *offs_s = reinterpret_cast<const float *>(st + St::OFFS);
         const uint4 *xb_s = reinterpret_cast<const uint4 *>(st + St::XB);
         const float *sx_s = reinterpret_cast<const float *>(st + St::SX);
-        (void)s;
-        constexpr bool with_offset = OFFSET && (T == T_Q5_1 || decltype(even_step)::value);
+        // this lane's row: 16 codes per group as two halves, scale and offset
+        uint4 frag[2][2];
+        float scr[2], ofr[2];
+        mm_decode<T, FB>(raw, s, frag, scr, ofr);
         bf16x8 wf[2][2];
         float sc[2][2], of[2][2];
 #pragma unroll
-        for (int g = 0; g < 2; g++)
-#pragma unroll
-            for (int rs = 0; rs < 2; rs++) {
-                const uint32_t r = wave * 64 + rs * 32 + n;
-                wf[g][rs] = __builtin_bit_cast(bf16x8, code_s[(2 * g + kh) * MM_ROWS + r]);
-                sc[g][rs] = scale_s[g * MM_ROWS + r];
-                of[g][rs] = OFFSET ? offs_s[g * MM_ROWS + r] : 0.f;
+        for (int g = 0; g < 2; g++) {
+            uint4 lo = frag[g][0], hi = frag[g][1];
+            swap32(lo.x, hi.x);
+            swap32(lo.y, hi.y);
+            swap32(lo.z, hi.z);
+            swap32(lo.w, hi.w);
+            wf[g][0] = __builtin_bit_cast(bf16x8, lo);  // rows 0..31 of the wavefront's 64: halves by lane / 32
+            wf[g][1] = __builtin_bit_cast(bf16x8, hi);  // rows 32..63
+            uint32_t s0 = __float_as_uint(scr[g]), s1 = s0;
+            swap32(s0, s1);
+            sc[g][0] = __uint_as_float(s0);
+            sc[g][1] = __uint_as_float(s1);
+            if constexpr (OFFSET) {
+                uint32_t o0 = __float_as_uint(ofr[g]), o1 = o0;
+                swap32(o0, o1);
+                of[g][0] = __uint_as_float(o0);
+                of[g][1] = __uint_as_float(o1);
+            } else {
+                of[g][0] = of[g][1] = 0.f;
             }
+        }
 #pragma unroll
         for (int tt = 0; tt < TT; tt++) {
             // one token tile at a time: interleaving the tiles only lengthens live ranges
@@ -1918,49 +1933,56 @@ __global__ __launch_bounds__(256, 2) void gemm_mfma_kernel(const MmBatch b) {
     };
 
     if (s_begin < s_end) {
-        // No branch inside a step: the compiler then knows how many loads are in flight
-        // and waits only for the oldest ring slot.  Step s computes from LDS stage
-        // (s - s_begin) & 1 while step s + 1 is decoded into the other stage from its
-        // ring slot, which is then refilled for step s + 1 + DEPTH.
-#define NH_MM_STEP(d, RAW, XB, SX)                                                     \
-    {                                                                                  \
-        store(base + d + 1, (d + 1) & 1, RAW, XB, SX);                                 \
-        fetch(base + d + 1 + DEPTH, RAW, XB, SX);                                      \
-        __builtin_amdgcn_sched_barrier(0);                                             \
-        compute(base + d, d & 1, std::integral_constant<bool, ((d) & 1) == 0>{});      \
-        __builtin_amdgcn_sched_barrier(0);                                             \
-        __syncthreads();                                                               \
+        // No branch inside a step: the compiler then knows how many loads are in flight and
+        // waits only for the oldest ring slot.  Step s reads its activations from LDS stage
+        // (s - s_begin) & 1; those of step s + 1 are written to the other stage meanwhile.
+#define NH_MM_STEP(d, RAW, XBN, SXN)                                                          \
+    {                                                                                          \
+        stage_x((d + 1) & 1, XBN, SXN);                                                        \
+        fetch_x(base + d + 1 + DEPTH, XBN, SXN);                                               \
+        const MmRaw<T> cur = RAW;                                                              \
+        fetch_w(base + d + DEPTH, RAW);                                                        \
+        __builtin_amdgcn_sched_barrier(0);                                                     \
+        compute(base + d, d & 1, cur, std::integral_constant<bool, ((d) & 1) == 0>{});         \
+        __builtin_amdgcn_sched_barrier(0);                                                     \
+        __syncthreads();                                                                       \
     }
         uint32_t base = s_begin;
         if constexpr (DEPTH == 4) {
-            fetch(s_begin, raw0, xb0, sx0);
-            fetch(s_begin + 1, raw1, xb1, sx1);
-            fetch(s_begin + 2, raw2, xb2, sx2);
-            fetch(s_begin + 3, raw3, xb3, sx3);
-            store(s_begin, 0, raw0, xb0, sx0);
-            fetch(s_begin + 4, raw0, xb0, sx0);
+            fetch_w(s_begin, raw0);
+            fetch_w(s_begin + 1, raw1);
+            fetch_w(s_begin + 2, raw2);
+            fetch_w(s_begin + 3, raw3);
+            fetch_x(s_begin, xb0, sx0);
+            fetch_x(s_begin + 1, xb1, sx1);
+            fetch_x(s_begin + 2, xb2, sx2);
+            fetch_x(s_begin + 3, xb3, sx3);
+            stage_x(0, xb0, sx0);
+            fetch_x(s_begin + 4, xb0, sx0);
             __syncthreads();
             for (; base + 4 <= s_end; base += 4) {
-                NH_MM_STEP(0, raw1, xb1, sx1)
-                NH_MM_STEP(1, raw2, xb2, sx2)
-                NH_MM_STEP(2, raw3, xb3, sx3)
-                NH_MM_STEP(3, raw0, xb0, sx0)
+                NH_MM_STEP(0, raw0, xb1, sx1)
+                NH_MM_STEP(1, raw1, xb2, sx2)
+                NH_MM_STEP(2, raw2, xb3, sx3)
+                NH_MM_STEP(3, raw3, xb0, sx0)
             }
             // at most three steps left (column counts that are not a multiple of 128)
-            if (base < s_end) NH_MM_STEP(0, raw1, xb1, sx1)
-            if (base + 1 < s_end) NH_MM_STEP(1, raw2, xb2, sx2)
-            if (base + 2 < s_end) NH_MM_STEP(2, raw3, xb3, sx3)
+            if (base < s_end) NH_MM_STEP(0, raw0, xb1, sx1)
+            if (base + 1 < s_end) NH_MM_STEP(1, raw1, xb2, sx2)
+            if (base + 2 < s_end) NH_MM_STEP(2, raw2, xb3, sx3)
         } else {
-            fetch(s_begin, raw0, xb0, sx0);
-            fetch(s_begin + 1, raw1, xb1, sx1);
-            store(s_begin, 0, raw0, xb0, sx0);
-            fetch(s_begin + 2, raw0, xb0, sx0);
+            fetch_w(s_begin, raw0);
+            fetch_w(s_begin + 1, raw1);
+            fetch_x(s_begin, xb0, sx0);
+            fetch_x(s_begin + 1, xb1, sx1);
+            stage_x(0, xb0, sx0);
+            fetch_x(s_begin + 2, xb0, sx0);
             __syncthreads();
             for (; base + 2 <= s_end; base += 2) {
-                NH_MM_STEP(0, raw1, xb1, sx1)
-                NH_MM_STEP(1, raw0, xb0, sx0)
+                NH_MM_STEP(0, raw0, xb1, sx1)
+                NH_MM_STEP(1, raw1, xb0, sx0)
             }
-            if (base < s_end) NH_MM_STEP(0, raw1, xb1, sx1)
+            if (base < s_end) NH_MM_STEP(0, raw0, xb1, sx1)
         }
 #undef NH_MM_STEP
     }
