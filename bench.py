@@ -40,6 +40,10 @@ sys.path.insert(0, ROOT)
 METRIC = "Q4_K/Q8_0 GEMV HBM GB/s (% of peak); 8B-shape decode tok/s, batch 1"
 HBM_PEAK_GBS = 8000.0
 BF16_MFMA_PEAK_TFLOPS = 2500.0
+# HBM bytes per Q4_K launch over algorithmic bytes, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this script (counters scaled by a 1 GiB copy kernel: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the
+# figures and commands are in profiles/decode_gemv_q4k_q6k_8b_step.txt.  Not measured by this run.
+Q4K_TRAFFIC_OVER_ALGORITHMIC = 1.0118
 Q4_0, Q8_0, Q4_K, Q6_K = 2, 8, 12, 14
 BLOCK = {Q4_0: (32, 18, 0), Q8_0: (32, 34, 0), Q4_K: (256, 144, 0), Q6_K: (256, 210, 208)}  # columns, bytes, offset of d
 N_LAYERS, D, D_KV, FF, VOCAB = 32, 4096, 1024, 14336, 128256
@@ -310,7 +314,9 @@ def main():
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "tok_per_s": round(args.steps / wall, 1),
         "roofline": {"bound": "hbm", "kernel": "gemv_q4k_kernel", "achieved": round(q4k_gbs, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(q4k_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(q4k_gbs / HBM_PEAK_GBS, 4),
+                     "traffic": round(Q4K_TRAFFIC_OVER_ALGORITHMIC * q4k_bytes / n_launch),
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiles/decode_gemv_q4k_q6k_8b_step.txt",
                      "bytes_per_launch": round(q4k_bytes / n_launch), "launch_us": round(q4k_launch_us, 3),
                      "launches_timed": args.steps * n_launch},
         "other_kernels": {"gemv_q6k_kernel (head)": {"achieved": round(head_gbs, 1), "unit": "GB/s",

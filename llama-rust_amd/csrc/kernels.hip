@@ -751,12 +751,6 @@ template <int LB> __device__ __forceinline__ float group_sum_dpp(float v) {
     return v;  // valid in the last lane of every group of LB lanes
 }
 
-#ifdef NH_TRACE
-__device__ unsigned long long nh_trace[8192 * 8];
-#define NH_T(slot) do { if (lane == 0) nh_trace[(size_t)(blockIdx.x * GEMV_WAVES + wave) * 8 + (slot)] = __builtin_readcyclecounter(); } while (0)
-#else
-#define NH_T(slot) do { } while (0)
-#endif
 
 // One unit of work of a lane: header and the eight 16-byte code pieces of its block.
 struct Q4kUnit {
@@ -820,7 +814,6 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b,
 
     uint32_t u = blockIdx.x * GEMV_WAVES + wave;
     Q4kUnit ua, ub;
-    NH_T(0);
     // Stage x once per workgroup; eight consecutive lanes hold one 32-column sub-block.
     // The x loads are issued before the first unit's weight loads, so they sit at the
     // head of the memory queue and the weights stream in behind them while x is
@@ -853,9 +846,7 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b,
             const uint32_t col = (tid + k * NW * 64) * 4;
             if (col < LB * 256) stage(col, col < cols ? xv[k] : make_float4(0.f, 0.f, 0.f, 0.f));
         }
-        NH_T(1);
         __syncthreads();
-        NH_T(2);
     } else {
         for (uint32_t col = tid * 4; col < n_iter * LB * 256; col += NW * 64 * 4)
             stage(col, col < cols ? *reinterpret_cast<const float4 *>(xw + col) : make_float4(0.f, 0.f, 0.f, 0.f));
@@ -914,12 +905,7 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b,
     while (u < n_units) {
         const uint32_t u2 = u + total_waves;
         if (u2 < n_units) fetch(u2, ub);
-#ifdef NH_TRACE
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        NH_T(3);
-#endif
         consume(u, ua);
-        NH_T(4);
         if (u2 >= n_units) break;
         u = u2 + total_waves;
         if (u < n_units) fetch(u, ua);
