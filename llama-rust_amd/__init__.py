@@ -56,6 +56,20 @@ def build(verbose=False):
     return LIB_PATH
 
 
+SELFTEST_SRC = os.path.join(os.path.dirname(HERE), "tests", "cpp", "selftest.cpp")
+SELFTEST_BIN = os.path.join(os.path.dirname(HERE), "tests", "cpp", "selftest")
+
+
+def build_selftest(verbose=False):
+    """Compile the C++ self-test (host code only: the C++ mirror header over the C ABI)."""
+    cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O2", "-Wall", "-Wextra", SELFTEST_SRC, "-o", SELFTEST_BIN,
+           "-L" + HERE, "-lnative_hip", "-Wl,-rpath,$ORIGIN/../../llama-rust_amd"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return SELFTEST_BIN
+
+
 _lib = None
 
 

@@ -130,3 +130,18 @@ def test_invalid_matrix_operations_preserve_output_without_touching_the_device(p
         pkg.gemv(pkg.Q8_0, 33, np.zeros(34, np.uint8), np.zeros(33, np.float32), np.zeros(1, np.float32))
     with pytest.raises(pkg.NativeHipError, match="unsupported GGUF dtype"):
         pkg.gemv(3, 32, np.zeros(20, np.uint8), np.zeros(32, np.float32), np.zeros(1, np.float32))
+
+
+def test_cpp_mirror_header_compiles_against_the_c_abi(pkg, tmp_path):
+    """include/native_hip.hpp (HipGemv, HipMatrix, Shape, validate over the C ABI) and the
+    self-test that uses it compile and link with the host compiler alone; running it needs a GPU
+    and is done by the GPU tests."""
+    import shutil
+    import subprocess
+    cxx = shutil.which(os.environ.get("CXX", "g++"))
+    if cxx is None:
+        pytest.skip("no host C++ compiler")
+    out = tmp_path / "selftest"
+    subprocess.run([cxx, "-std=c++17", "-Wall", "-Wextra", "-Werror", pkg.SELFTEST_SRC, "-o", str(out), "-L" + pkg.HERE,
+                    "-lnative_hip"], check=True)
+    assert out.exists()

@@ -18,6 +18,8 @@ dequantized weights:
         as e -> 0 for ANY f32 summation order, the reference's CPU kernels
         included, because the rounding error scales with sum|w x|, not with |e|).
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -59,6 +61,16 @@ def check(actual, ty, n_cols, n_tokens, n_rows, w, x, name="", strict=False):
 
 
 # ------------------------------------------------------------------ native-cuda/src/main.rs
+def test_cpp_selftest_through_the_mirror_header(pkg):
+    """The same scenario from C++ (tests/cpp/selftest.cpp over include/native_hip.hpp): a
+    maintainer's compiled host code reaches the kernels through the C ABI only."""
+    import subprocess
+    if not os.path.exists(pkg.SELFTEST_BIN):
+        pkg.build_selftest()
+    r = subprocess.run([pkg.SELFTEST_BIN], capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0 and r.stdout.startswith("OK"), r.stdout + r.stderr
+
+
 def test_executor_selftest_shapes_and_rounds(pkg, gpu):
     """native-cuda/src/main.rs:8-45: revisited shapes, alternating vector/batch launches,
     every equal-sized reuse changes all inputs, every output is checked."""
