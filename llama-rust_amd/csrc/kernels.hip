@@ -2360,7 +2360,14 @@ static hipError_t launch_multi_t(hipStream_t stream, const MatView *mats, float 
         if (e != hipErrorInvalidValue) return e;
         (void)hipGetLastError();
     }
-    return launch_gemv_t<T, 4>(stream, mats, ys, n, x);
+    // Rows per lane: four share the lane's activations, but a wavefront owns whole row groups, so
+    // matrices with few rows take fewer rows per group to give every wavefront of the chip one.
+    size_t rows = 0;
+    for (uint32_t j = 0; j < n; j++) rows += mats[j].rows;
+    const size_t wavefronts = (size_t)g_cu_count * 16;
+    if (rows >= 4 * wavefronts) return launch_gemv_t<T, 4>(stream, mats, ys, n, x);
+    if (rows >= 2 * wavefronts) return launch_gemv_t<T, 2>(stream, mats, ys, n, x);
+    return launch_gemv_t<T, 1>(stream, mats, ys, n, x);
 }
 
 // ---- MFMA GEMM: planning and launch
