@@ -752,24 +752,32 @@ template <int LB> __device__ __forceinline__ float group_sum_dpp(float v) {
 }
 
 
-// One unit of work of a lane: header and the eight 16-byte code pieces of its block.
-struct Q4kUnit {
-    uint4 hdr, q[8];
+// One unit of work of a lane: the header of its block and PL of its eight 16-byte code pieces.
+template <int PL> struct Q4kUnit {
+    uint4 hdr, q[PL];
 };
 
-template <int LB, int NW, bool FP8>
+// PL = 8: a lane owns a whole super-block.  PL = 4: two lanes share one (pieces 0..3 = sub-blocks
+// 0..3, pieces 4..7 = sub-blocks 4..7), which doubles the wavefronts a short-row matrix gives the
+// chip and halves the arithmetic left to do after a wavefront's last bytes have arrived.
+// LB lanes cover a row: LB / (8 / PL) blocks, the first half of the lanes holding the first halves.
+template <int LB, int NW, bool FP8, int PL>
 __global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b, const float nib_mul) {
     constexpr int GEMV_WAVES = NW;  // wavefronts per workgroup of this instantiation
     constexpr uint32_t RS = 64 / LB;       // rows per wavefront step = rows per row group
+    constexpr uint32_t HALVES = 8 / PL;    // lanes per super-block
+    constexpr uint32_t LBB = LB / HALVES;  // super-blocks per row and iteration
+    static_assert(PL == 8 || PL == 4, "a lane owns a whole super-block or half of one");
+    static_assert(LB >= HALVES, "too few lanes per row for half blocks");
     // LDS row of one (cc, i) slot: LB float4 plus one float4 of padding, so that the 16 slots
     // consecutive staging lanes write to fall into different banks.
-    constexpr uint32_t XROW = LB * 4 + 4;
+    constexpr uint32_t XROW = LBB * 4 + 4;
     constexpr uint32_t XS_FLOATS = 64 * XROW;  // x region of one block iteration
     extern __shared__ __align__(16) float lds[];
     const uint32_t nb_all = b.job[0].m.nb;         // super-blocks per row: slot stride of the piece-major plane
     const uint32_t nb = b.units, cols = nb * 256;  // the window this launch covers
     const float *xw = b.x + (size_t)b.unit0 * 256;
-    const uint32_t n_iter = (nb + LB - 1) / LB;    // always 1: the launcher cuts windows of at most 64 super-blocks
+    const uint32_t n_iter = (nb + LBB - 1) / LBB;  // always 1: the launcher cuts windows of at most LBB super-blocks
     // x, permuted so that lane blk reads piece i of code piece cc at a compile-time offset:
     //   float it * XS_FLOATS + (cc*8 + i) * XROW + (blk % LB) * 4 + e,   it = blk / LB
     float *xs = lds;
@@ -779,6 +787,7 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b,
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t total_waves = gridDim.x * GEMV_WAVES;
     const uint32_t sub_row = lane / LB, b0 = lane % LB;
+    const uint32_t bl0 = b0 % LBB, half = b0 / LBB;  // block of the iteration, which half of it
     const uint32_t n_units = b.total_rgs * n_iter;  // unit u = (row group u / n_iter, iteration u % n_iter)
 
     struct Where {
@@ -799,28 +808,29 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b,
         w.row0 = (g - b.job[j].rg_begin) * RS;
         return w;
     };
-    auto fetch = [&](uint32_t u, Q4kUnit &o) {
+    auto fetch = [&](uint32_t u, Q4kUnit<PL> &o) {
         const uint32_t g = u / n_iter, it = u - g * n_iter;
         const Where w = locate(g);
         uint32_t row = w.row0 + sub_row;
         row = row < w.rows ? row : w.rows - 1;
-        uint32_t blk = it * LB + b0;
+        uint32_t blk = it * LBB + bl0;
         blk = b.unit0 + (blk < nb ? blk : nb - 1);
         const uint32_t hoff = row * w.s1 + blk * 16, qoff = row * w.s0 + blk * 16;  // planes stay below 4 GB
         o.hdr = *reinterpret_cast<const uint4 *>(w.p1 + hoff);
 #pragma unroll
-        for (int cc = 0; cc < 8; cc++) o.q[cc] = *reinterpret_cast<const uint4 *>(w.p0 + (size_t)cc * nb_all * 16 + qoff);
+        for (int c = 0; c < PL; c++)
+            o.q[c] = *reinterpret_cast<const uint4 *>(w.p0 + (size_t)(half * PL + c) * nb_all * 16 + qoff);
     };
 
     uint32_t u = blockIdx.x * GEMV_WAVES + wave;
-    Q4kUnit ua, ub;
+    Q4kUnit<PL> ua, ub;
     // Stage x once per workgroup; eight consecutive lanes hold one 32-column sub-block.
     // The x loads are issued before the first unit's weight loads, so they sit at the
     // head of the memory queue and the weights stream in behind them while x is
     // being written to LDS.
     auto stage = [&](uint32_t col, const float4 v) {
         const uint32_t blk = col >> 8, r = col & 255u, g = r >> 6, r2 = r & 63u, hi = r2 >> 5, r3 = r2 & 31u;
-        const uint32_t cc = 2 * g + (r3 >> 4), t = hi * 16 + (r3 & 15u), it = blk / LB, bl = blk % LB;
+        const uint32_t cc = 2 * g + (r3 >> 4), t = hi * 16 + (r3 & 15u), it = blk / LBB, bl = blk % LBB;
         *reinterpret_cast<float4 *>(xs + (size_t)it * XS_FLOATS + (cc * 8 + (t >> 2)) * XROW + bl * 4) = v;
         float sm = (v.x + v.y) + (v.z + v.w);
 #define NH_DPP_ADD(ctrl) sm += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), ctrl, 0xf, 0xf, false))
@@ -828,9 +838,9 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b,
         NH_DPP_ADD(0x4e);
         NH_DPP_ADD(0x141);
 #undef NH_DPP_ADD
-        if ((lane & 7u) == 0) ssum[(it * 8 + (r >> 5)) * LB + bl] = sm;
+        if ((lane & 7u) == 0) ssum[(it * 8 + (r >> 5)) * LBB + bl] = sm;
     };
-    constexpr int NXV = (LB * 64 + NW * 64 - 1) / (NW * 64);  // float4 per thread for LB blocks of x
+    constexpr int NXV = (LBB * 64 + NW * 64 - 1) / (NW * 64);  // float4 per thread for LBB blocks of x
     if (n_iter == 1) {
         float4 xv[NXV];
 #pragma unroll
@@ -844,51 +854,67 @@ __global__ __launch_bounds__(NW * 64, 4) void gemv_q4k_kernel(const GemvBatch b,
 #pragma unroll
         for (int k = 0; k < NXV; k++) {
             const uint32_t col = (tid + k * NW * 64) * 4;
-            if (col < LB * 256) stage(col, col < cols ? xv[k] : make_float4(0.f, 0.f, 0.f, 0.f));
+            if (col < LBB * 256) stage(col, col < cols ? xv[k] : make_float4(0.f, 0.f, 0.f, 0.f));
         }
         __syncthreads();
     } else {
-        for (uint32_t col = tid * 4; col < n_iter * LB * 256; col += NW * 64 * 4)
+        for (uint32_t col = tid * 4; col < n_iter * LBB * 256; col += NW * 64 * 4)
             stage(col, col < cols ? *reinterpret_cast<const float4 *>(xw + col) : make_float4(0.f, 0.f, 0.f, 0.f));
         __syncthreads();
         if (u < n_units) fetch(u, ua);
     }
 
     float acc = 0.f;
-    auto consume = [&](uint32_t uu, const Q4kUnit &q) {
+    auto consume = [&](uint32_t uu, const Q4kUnit<PL> &q) {
         const uint32_t g = uu / n_iter, it = uu - g * n_iter;
-        const bool active = it * LB + b0 < nb;
-        const float *xb = xs + (size_t)it * XS_FLOATS + b0 * 4;
-        float t[8];
+        const bool active = it * LBB + bl0 < nb;
+        // x rows of this lane's pieces: piece cc = half * PL + c starts at row cc * 8
+        const float *xb = xs + (size_t)it * XS_FLOATS + bl0 * 4 + half * (PL * 8 * XROW);
+        float t[PL];
 #pragma unroll
-        for (int k = 0; k < 8; k++) t[k] = 0.f;
+        for (int k = 0; k < PL; k++) t[k] = 0.f;
 #pragma unroll
-        for (int cc = 0; cc < 8; cc++) {
+        for (int c = 0; c < PL; c++) {
             float x[32];
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                float4 v = *reinterpret_cast<const float4 *>(xb + (cc * 8 + i) * XROW);
+                float4 v = *reinterpret_cast<const float4 *>(xb + (c * 8 + i) * XROW);
                 x[4 * i] = v.x; x[4 * i + 1] = v.y; x[4 * i + 2] = v.z; x[4 * i + 3] = v.w;
             }
-            const uint32_t w[4] = {q.q[cc].x, q.q[cc].y, q.q[cc].z, q.q[cc].w};
+            const uint32_t w[4] = {q.q[c].x, q.q[c].y, q.q[c].z, q.q[c].w};
 #pragma unroll
             for (int d = 0; d < 4; d++) {
-                t[cc & ~1] = dot4_nib<FP8>(w[d] & 0x0f0f0f0fu, x + 4 * d, t[cc & ~1]);
-                t[cc | 1] = dot4_nib<FP8>((w[d] >> 4) & 0x0f0f0f0fu, x + 16 + 4 * d, t[cc | 1]);
+                t[c & ~1] = dot4_nib<FP8>(w[d] & 0x0f0f0f0fu, x + 4 * d, t[c & ~1]);
+                t[c | 1] = dot4_nib<FP8>((w[d] >> 4) & 0x0f0f0f0fu, x + 16 + 4 * d, t[c | 1]);
             }
         }
         const uint32_t h1 = q.hdr.y, h2 = q.hdr.z, h3 = q.hdr.w;
-        const float *sp = ssum + (size_t)it * 8 * LB + b0;
         float S = 0.f, Mn = 0.f;
+        if constexpr (PL == 8) {
+            const float *sp = ssum + (size_t)it * 8 * LBB + bl0;
 #pragma unroll
-        for (int k = 0; k < 4; k++) {  // langtax/src/quant.rs:8901-8912 with constant shifts
-            const float sc_lo = (float)((h1 >> (8 * k)) & 63u), mn_lo = (float)((h2 >> (8 * k)) & 63u);
-            const float sc_hi = (float)(((h3 >> (8 * k)) & 15u) | (((h1 >> (8 * k + 6)) & 3u) << 4));
-            const float mn_hi = (float)(((h3 >> (8 * k + 4)) & 15u) | (((h2 >> (8 * k + 6)) & 3u) << 4));
-            S = fmaf(sc_lo, t[k], S);
-            S = fmaf(sc_hi, t[k + 4], S);
-            Mn = fmaf(mn_lo, sp[k * LB], Mn);
-            Mn = fmaf(mn_hi, sp[(k + 4) * LB], Mn);
+            for (int k = 0; k < 4; k++) {  // langtax/src/quant.rs:8901-8912 with constant shifts
+                const float sc_lo = (float)((h1 >> (8 * k)) & 63u), mn_lo = (float)((h2 >> (8 * k)) & 63u);
+                const float sc_hi = (float)(((h3 >> (8 * k)) & 15u) | (((h1 >> (8 * k + 6)) & 3u) << 4));
+                const float mn_hi = (float)(((h3 >> (8 * k + 4)) & 15u) | (((h2 >> (8 * k + 6)) & 3u) << 4));
+                S = fmaf(sc_lo, t[k], S);
+                S = fmaf(sc_hi, t[k + 4], S);
+                Mn = fmaf(mn_lo, sp[k * LBB], Mn);
+                Mn = fmaf(mn_hi, sp[(k + 4) * LBB], Mn);
+            }
+        } else {
+            // sub-blocks 4 half .. 4 half + 3: the first half's pairs sit whole in the header, the
+            // second half's are split over its three dwords
+            const float *sp = ssum + ((size_t)it * 8 + 4 * half) * LBB + bl0;
+            const uint32_t up = 0u - half;  // all ones in the second half
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const uint32_t sc_lo = (h1 >> (8 * k)) & 63u, mn_lo = (h2 >> (8 * k)) & 63u;
+                const uint32_t sc_hi = ((h3 >> (8 * k)) & 15u) | (((h1 >> (8 * k + 6)) & 3u) << 4);
+                const uint32_t mn_hi = ((h3 >> (8 * k + 4)) & 15u) | (((h2 >> (8 * k + 6)) & 3u) << 4);
+                S = fmaf((float)(sc_lo ^ ((sc_lo ^ sc_hi) & up)), t[k], S);
+                Mn = fmaf((float)(mn_lo ^ ((mn_lo ^ mn_hi) & up)), sp[k * LBB], Mn);
+            }
         }
         const float d = h2f((uint16_t)(q.hdr.x & 0xffffu)) * nib_mul, dmin = h2f((uint16_t)(q.hdr.x >> 16));
         const float part = fmaf(d, S, -(dmin * Mn));
@@ -2143,11 +2169,11 @@ hipError_t probe_fp8_nibble_unit(hipStream_t stream, float *unit_out) {
 static float g_nib_mul = 0.f;  // 1 / (value of fp8 byte 0x01); 0 = fp8 unpack not usable
 void set_fp8_nibble_unit(float unit) { g_nib_mul = unit > 0.f ? 1.0f / unit : 0.f; }
 
-template <int LB, int NW>
+template <int LB, int NW, int PL>
 static hipError_t launch_q4k_lb(hipStream_t stream, const GemvBatch &b, uint32_t units, size_t lds) {
     const bool fp8 = g_nib_mul != 0.f;
-    const void *kern = fp8 ? reinterpret_cast<const void *>(gemv_q4k_kernel<LB, NW, true>)
-                           : reinterpret_cast<const void *>(gemv_q4k_kernel<LB, NW, false>);
+    const void *kern = fp8 ? reinterpret_cast<const void *>(gemv_q4k_kernel<LB, NW, true, PL>)
+                           : reinterpret_cast<const void *>(gemv_q4k_kernel<LB, NW, false, PL>);
     static size_t configured[2] = {0, 0};
     if (lds > 48 * 1024 && lds > configured[fp8]) {
         hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g_lds_limit);
@@ -2162,9 +2188,9 @@ static hipError_t launch_q4k_lb(hipStream_t stream, const GemvBatch &b, uint32_t
     if (grid > needed) grid = needed;
     const float mul = fp8 ? g_nib_mul : 1.0f;
     if (fp8)
-        hipLaunchKernelGGL((gemv_q4k_kernel<LB, NW, true>), dim3(grid), dim3(NW * 64), lds, stream, b, mul);
+        hipLaunchKernelGGL((gemv_q4k_kernel<LB, NW, true, PL>), dim3(grid), dim3(NW * 64), lds, stream, b, mul);
     else
-        hipLaunchKernelGGL((gemv_q4k_kernel<LB, NW, false>), dim3(grid), dim3(NW * 64), lds, stream, b, mul);
+        hipLaunchKernelGGL((gemv_q4k_kernel<LB, NW, false, PL>), dim3(grid), dim3(NW * 64), lds, stream, b, mul);
     return hipGetLastError();
 }
 
@@ -2206,25 +2232,41 @@ static hipError_t launch_gemv_q4k(hipStream_t stream, const MatView *mats, float
     const UnitWindows win(nb, 64);
     for (uint32_t w = 0; w < win.n; w++) {
         const uint32_t units = win.count(w, nb);
-        uint32_t lb = 1;
-        while (lb < 64 && lb < units) lb <<= 1;
+        uint32_t lbb = 1;  // super-blocks per row, rounded up to a power of two
+        while (lbb < 64 && lbb < units) lbb <<= 1;
+        // Two lanes per super-block for matrices that would otherwise give the chip fewer than about ten
+        // wavefront steps per CU (measured crossover: 8192 x 4096 gains 11 %, 12288 x 4096 loses 6 %).
+        size_t full_steps = 0;
+        for (uint32_t j = 0; j < n_jobs; j++) full_steps += (mats[j].rows + 64 / lbb - 1) / (64 / lbb);
+        const bool halves = lbb <= 16 && full_steps <= (size_t)10 * g_cu_count;
+        const uint32_t lb = halves ? 2 * lbb : lbb;
         GemvBatch b;
         const uint32_t rgs = fill_unit_jobs(b, mats, ys, n_jobs, x, lb);
         b.unit0 = win.first(w);
         b.units = units;
         b.accumulate = w > 0;
-        const size_t lds = (size_t)(64 * (lb * 4 + 4) + lb * 8) * sizeof(float);
+        const size_t lds = (size_t)(64 * (lbb * 4 + 4) + lbb * 8) * sizeof(float);
         if (lds > g_lds_limit) return hipErrorInvalidValue;
         hipError_t e;
-        switch (lb) {
-        // Short rows: small workgroups, so that even a 1024-row matrix spreads over every CU.
-        case 1: e = launch_q4k_lb<1, 4>(stream, b, rgs, lds); break;
-        case 2: e = launch_q4k_lb<2, 4>(stream, b, rgs, lds); break;
-        case 4: e = launch_q4k_lb<4, 4>(stream, b, rgs, lds); break;
-        case 8: e = launch_q4k_lb<8, 4>(stream, b, rgs, lds); break;
-        case 16: e = launch_q4k_lb<16, 4>(stream, b, rgs, lds); break;
-        case 32: e = launch_q4k_lb<32, 8>(stream, b, rgs, lds); break;
-        default: e = launch_q4k_lb<64, 8>(stream, b, rgs, lds); break;
+        if (halves) {
+            switch (lb) {
+            case 2: e = launch_q4k_lb<2, 4, 4>(stream, b, rgs, lds); break;
+            case 4: e = launch_q4k_lb<4, 4, 4>(stream, b, rgs, lds); break;
+            case 8: e = launch_q4k_lb<8, 4, 4>(stream, b, rgs, lds); break;
+            case 16: e = launch_q4k_lb<16, 4, 4>(stream, b, rgs, lds); break;
+            default: e = launch_q4k_lb<32, 4, 4>(stream, b, rgs, lds); break;
+            }
+        } else {
+            switch (lb) {
+            // Short rows: small workgroups, so that even a 1024-row matrix spreads over every CU.
+            case 1: e = launch_q4k_lb<1, 4, 8>(stream, b, rgs, lds); break;
+            case 2: e = launch_q4k_lb<2, 4, 8>(stream, b, rgs, lds); break;
+            case 4: e = launch_q4k_lb<4, 4, 8>(stream, b, rgs, lds); break;
+            case 8: e = launch_q4k_lb<8, 4, 8>(stream, b, rgs, lds); break;
+            case 16: e = launch_q4k_lb<16, 4, 8>(stream, b, rgs, lds); break;
+            case 32: e = launch_q4k_lb<32, 8, 8>(stream, b, rgs, lds); break;
+            default: e = launch_q4k_lb<64, 8, 8>(stream, b, rgs, lds); break;
+            }
         }
         if (e != hipSuccess) return e;
     }
