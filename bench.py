@@ -122,10 +122,25 @@ def timed_us(hip, stream, enqueue, n_variants, reps):
     return a.elapsed_ms(b) * 1e3 / (reps * n_variants)
 
 
-def other_workloads(pkg, hip, gpu, stream, rng):
-    """Shapes of the reference's other benchmark configurations (see the module docstring)."""
+def other_workloads(pkg, hip, gpu, stream, rng, cpu):
+    """Shapes of the reference's other benchmark configurations (see the module docstring).
+    With `cpu`, each entry also carries the AVX2 port of the reference's CPU kernels on a sample of
+    the same product's rows (its threading rule, all tokens), scaled to the whole product."""
     import oracle as O
     out = {}
+
+    def cpu_us(ty, rows, cols, tokens, w, x, sample_rows):
+        """Microseconds the CPU path would take for the whole product, from `sample_rows` rows."""
+        if not cpu:
+            return None
+        ws = w[:sample_rows * row_bytes(ty, cols)]
+        O.gemm(ty, cols, tokens, ws, x, sample_rows, simd=True, threads=0)  # warm-up
+        t0 = time.perf_counter()
+        n = 0
+        while n < 3 or time.perf_counter() - t0 < 0.3:
+            O.gemm(ty, cols, tokens, ws, x, sample_rows, simd=True, threads=0)
+            n += 1
+        return round((time.perf_counter() - t0) / n * 1e6 * rows / sample_rows, 1)
 
     def check(name, ty, rows, cols, tokens, w, x, y_dev):
         got = y_dev.to_numpy(np.float32)[:tokens * rows].reshape(tokens, rows)[:, :32]
@@ -145,7 +160,8 @@ def other_workloads(pkg, hip, gpu, stream, rng):
     check("Q8_0 GEMV", Q8_0, D, D, 1, ws[0], x, yd)
     nbytes = algorithmic_bytes(Q8_0, D, D)
     out["gemv_q8_0_4096x4096"] = {"launch_us": round(us, 2), "achieved": round(nbytes / us / 1e3, 1), "unit": "GB/s",
-                                  "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "bound": "hbm"}
+                                  "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "bound": "hbm",
+                                  "cpu_us": cpu_us(Q8_0, D, D, 1, ws[0], x, D)}
     for m in ms:
         m.close()
 
@@ -164,7 +180,8 @@ def other_workloads(pkg, hip, gpu, stream, rng):
         out[f"gemm_q4_0_4096x14336_m{tokens}"] = {
             "call_us": round(us, 2), "tflops": round(flops / us / 1e6, 1),
             "mfma_frac": round(3 * flops / us / 1e6 / BF16_MFMA_PEAK_TFLOPS, 4),
-            "weight_gbs": round(D * row_bytes(Q4_0, FF) / us / 1e3, 1), "bound": "mfma" if tokens >= 128 else "hbm"}
+            "weight_gbs": round(D * row_bytes(Q4_0, FF) / us / 1e3, 1), "bound": "mfma" if tokens >= 128 else "hbm",
+            "cpu_us": cpu_us(Q4_0, D, FF, tokens, ws[0], x[:tokens * FF], 256 if tokens >= 128 else D)}
     for m in ms:
         m.close()
 
@@ -181,7 +198,8 @@ def other_workloads(pkg, hip, gpu, stream, rng):
     wbytes = n_exp * FF * row_bytes(Q4_K, D)
     out["moe_q4_k_8x14336x4096_m16"] = {"call_us": round(us, 2), "weight_gbs": round(wbytes / us / 1e3, 1),
                                          "frac": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4),
-                                         "tflops": round(2.0 * n_exp * per * FF * D / us / 1e6, 1), "bound": "hbm"}
+                                         "tflops": round(2.0 * n_exp * per * FF * D / us / 1e6, 1), "bound": "hbm",
+                                         "cpu_us": None if not cpu else round(n_exp * cpu_us(Q4_K, FF, D, per, ws[0][0], x[:per * D], 2048), 1)}
     for ms_ in ms:
         for m in ms_:
             m.close()
@@ -328,7 +346,7 @@ def main():
         for m in mats:
             m.close()
         head.close()
-        out["other_workloads"] = other_workloads(pkg, hip, gpu, stream, rng)
+        out["other_workloads"] = other_workloads(pkg, hip, gpu, stream, rng, args.cpu_seconds > 0)
     if args.cpu_seconds > 0:
         log("[bench] timing the CPU baseline ...")
         out["cpu_baseline"] = cpu_baseline(sample, x_host, args.cpu_seconds)
