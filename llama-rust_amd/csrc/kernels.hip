@@ -290,7 +290,7 @@ static hipError_t launch_gemv_q6k(hipStream_t stream, const MatView *mats, float
         case 8: e = launch_q6k_lb<8, 4>(stream, b, rgs, lds); break;
         case 16: e = launch_q6k_lb<16, 4>(stream, b, rgs, lds); break;
         case 32: e = launch_q6k_lb<32, 8>(stream, b, rgs, lds); break;
-        default: e = launch_q6k_lb<64, 8>(stream, b, rgs, lds); break;
+        default: e = launch_q6k_lb<64, 16>(stream, b, rgs, lds); break;  // measured 7 % faster than 8 wavefronts
         }
         if (e != hipSuccess) return e;
     }
@@ -354,7 +354,9 @@ static hipError_t launch_gemv_b32(hipStream_t stream, const MatView *mats, float
         case 8: e = launch_b32_lb<T, 8, 4>(stream, b, rgs, lds); break;
         case 16: e = launch_b32_lb<T, 16, 4>(stream, b, rgs, lds); break;
         case 32: e = launch_b32_lb<T, 32, 8>(stream, b, rgs, lds); break;
-        default: e = launch_b32_lb<T, 64, 8>(stream, b, rgs, lds); break;
+        default:  // 16 wavefronts per workgroup measured 3 % faster for Q8_0, 12 % slower for the nibble dtypes
+            e = T == T_Q8_0 ? launch_b32_lb<T, 64, 16>(stream, b, rgs, lds) : launch_b32_lb<T, 64, 8>(stream, b, rgs, lds);
+            break;
         }
         if (e != hipSuccess) return e;
     }
