@@ -146,25 +146,25 @@ void set_fp8_nibble_unit(float unit) { g_nib_mul = unit > 0.f ? 1.0f / unit : 0.
 template <int LB, int NW, int PL>
 static hipError_t launch_q4k_lb(hipStream_t stream, const GemvBatch &b, uint32_t units, size_t lds) {
     const bool fp8 = g_nib_mul != 0.f;
-    const void *kern = fp8 ? reinterpret_cast<const void *>(gemv_q4k_kernel<LB, NW, true, PL>)
-                           : reinterpret_cast<const void *>(gemv_q4k_kernel<LB, NW, false, PL>);
-    static size_t configured[2] = {0, 0};
-    if (lds > 48 * 1024 && lds > configured[fp8]) {
-        hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g_lds_limit);
-        if (e != hipSuccess) return e;
-        configured[fp8] = g_lds_limit;
-    }
     size_t per_cu = g_lds_limit * 2 / (lds ? lds : 1);  // 160 KB of LDS per CU
     if (per_cu < 1) per_cu = 1;
-    if (per_cu > 32 / NW) per_cu = 32 / NW;             // 32 wavefronts per CU (64 VGPRs each; measured +2.5 % on the decode step over 16)
+    if (per_cu > 32 / NW) per_cu = 32 / NW;             // 32 wavefronts per CU (measured +2.5 % on the decode step over 16)
     uint32_t grid = (uint32_t)((size_t)g_cu_count * per_cu);
     const uint32_t needed = (units + NW - 1) / NW;
     if (grid > needed) grid = needed;
-    const float mul = fp8 ? g_nib_mul : 1.0f;
-    if (fp8)
-        hipLaunchKernelGGL((gemv_q4k_kernel<LB, NW, true, PL>), dim3(grid), dim3(NW * 64), lds, stream, b, mul);
-    else
-        hipLaunchKernelGGL((gemv_q4k_kernel<LB, NW, false, PL>), dim3(grid), dim3(NW * 64), lds, stream, b, mul);
+    const bool one = grid == needed;  // a wavefront for every unit
+    void (*kern)(GemvBatch, float) =
+        fp8 ? (one ? gemv_q4k_kernel<LB, NW, true, PL, true> : gemv_q4k_kernel<LB, NW, true, PL, false>)
+            : (one ? gemv_q4k_kernel<LB, NW, false, PL, true> : gemv_q4k_kernel<LB, NW, false, PL, false>);
+    static size_t configured[4] = {0, 0, 0, 0};
+    size_t &conf = configured[2 * fp8 + one];
+    if (lds > 48 * 1024 && lds > conf) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)g_lds_limit);
+        if (e != hipSuccess) return e;
+        conf = g_lds_limit;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, stream, b, fp8 ? g_nib_mul : 1.0f);
     return hipGetLastError();
 }
 
