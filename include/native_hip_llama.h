@@ -1,0 +1,104 @@
+/*
+ * native-hip, host side of a dense Llama decode: the caller of the matrix products.
+ *
+ * The matrix executor (native_hip.h) replaces one seam of the reference; this header is
+ * the code either side of that seam, restated in C++ so that an end-to-end greedy decode
+ * of a GGUF model can run and be checked without the reference's Rust toolchain:
+ *
+ *   GGUF v3 reader / writer             langtax/src/gguf.rs:64-68, 626-702, 728-828, 922-947
+ *   model load (llama architecture)     langtax/src/decode.rs:1910-1958, 2050-2090, 7461-7475
+ *   forward pass of n tokens            langtax/src/decode.rs:2710-3099 (dense llama branch)
+ *     RMSNorm 11498-11513, RoPE (adjacent pairs) 11578-11602, attention 11126-11197,
+ *     softmax 12021-12033, SiLU 11826-11830, argmax 12104-12114, embedding 10761-10800
+ *   paged K/V addressing                langtax/src/kv_page.rs:410-438, decode.rs:12059-12100
+ *
+ * All host arithmetic is f32 in the reference's operation order.  Every weight product
+ * goes through one of three routes, chosen per model:
+ *   LNM_PRODUCTS_RESIDENT  matrices uploaded once (lnh_upload_packed), products by lnh_gemm
+ *   LNM_PRODUCTS_DISPATCH  lnq_gemv / lnq_gemm, i.e. the reference's call shape with the
+ *                          content-identified residency cache behind it
+ *   LNM_PRODUCTS_CALLBACK  a function of the caller (tests plug their CPU checker in here;
+ *                          the library itself contains no CPU implementation of a product)
+ *
+ * Errors: every call returns 0 on success; otherwise a non-zero code with the text in
+ * lnm_last_error() (thread-local, valid until the next lnm call on the thread).
+ */
+#ifndef NATIVE_HIP_LLAMA_H
+#define NATIVE_HIP_LLAMA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct lnm_model lnm_model;
+typedef struct lnm_session lnm_session;
+
+typedef struct lnm_hparams {
+    uint32_t n_layer, n_embd, n_head, n_head_kv, n_ff, n_vocab, head_dim, n_rot;
+    float rope_base, rms_eps;
+    uint32_t block_type, embd_type, output_type; /* ggml type ids of blk.0.attn_q, token_embd, output */
+} lnm_hparams;
+
+enum { LNM_PRODUCTS_RESIDENT = 0, LNM_PRODUCTS_DISPATCH = 1, LNM_PRODUCTS_CALLBACK = 2 };
+
+/* y[t * n_rows + r] = sum_c W[r, c] * x[t * n_cols + c]; returns 0 on success. */
+typedef int (*lnm_matmul_fn)(void *user, uint32_t ggml_type, size_t n_rows, size_t n_cols, size_t n_tokens,
+                             const uint8_t *w, size_t w_len, const float *x, float *y);
+
+const char *lnm_last_error(void);
+
+/* Maps the file and validates the llama hyper-parameters and tensor shapes. */
+int lnm_load(const char *gguf_path, lnm_model **out);
+/* Same from memory; the bytes are copied. */
+int lnm_load_bytes(const uint8_t *bytes, size_t len, lnm_model **out);
+void lnm_free(lnm_model *model);
+int lnm_info(const lnm_model *model, lnm_hparams *out);
+/* Route of the products; `fn` and `user` are used by LNM_PRODUCTS_CALLBACK only.  Default: RESIDENT. */
+int lnm_set_products(lnm_model *model, int route, lnm_matmul_fn fn, void *user);
+
+/* One sequence with a paged K/V cache of `kv_block` positions per block.  `block_ids` (may be
+ * NULL) gives the physical block of each logical block, any permutation of 0 .. n_block_ids-1;
+ * NULL allocates blocks in order as the sequence grows. */
+int lnm_session_new(lnm_model *model, size_t kv_block, const uint32_t *block_ids, size_t n_block_ids,
+                    lnm_session **out);
+void lnm_session_free(lnm_session *session);
+/* Runs the n tokens as one batch at positions past .. past+n-1 (products with n_tokens = n) and
+ * writes the logits of the last one (n_vocab floats). */
+int lnm_forward(lnm_session *session, const uint32_t *tokens, size_t n, float *logits);
+/* Greedy decode: the prompt as one batch, then one token at a time; out[0] comes from the prompt's
+ * logits, out[i] from decode step i, n_new tokens and n_new - 1 decode steps in all.  The two
+ * wall times (seconds) may be NULL. */
+int lnm_generate_greedy(lnm_session *session, const uint32_t *prompt, size_t n_prompt, size_t n_new,
+                        uint32_t *out, double *prefill_seconds, double *decode_seconds);
+
+/* Building blocks, exported so that each can be checked on its own. */
+int lnm_dequant_row(uint32_t ggml_type, size_t n_cols, const uint8_t *row, size_t row_len, float *y);
+int lnm_rmsnorm(float *x, const float *w, size_t n, float eps);
+int lnm_rope(float *head, size_t head_len, size_t pos, size_t n_rot, float base);
+void lnm_softmax(float *x, size_t n);
+uint32_t lnm_argmax(const float *x, size_t n);
+
+/* A random dense llama model written as GGUF v3: packed blocks are drawn directly (codes uniform,
+ * block scales sized so that the dequantized weights have mean 0 and standard deviation
+ * `weight_std`), norm weights are 1 + N(0, 0.05).  Deterministic in `seed`. */
+typedef struct lnm_synth_spec {
+    uint32_t n_layer, n_embd, n_head, n_head_kv, n_ff, n_vocab;
+    uint32_t block_type, embd_type, output_type; /* ggml type ids */
+    float rope_base, rms_eps, weight_std;
+    uint64_t seed;
+} lnm_synth_spec;
+int lnm_write_synthetic_llama(const char *gguf_path, const lnm_synth_spec *spec);
+
+/* GGUF container checks without a model: number of tensors and keys, or an error. */
+int lnm_gguf_inspect(const uint8_t *bytes, size_t len, size_t *n_tensors, size_t *n_kv, size_t *alignment);
+/* Tensor i of a GGUF blob: name (copied, NUL-terminated, truncated to name_cap), type, dims, byte range. */
+int lnm_gguf_tensor(const uint8_t *bytes, size_t len, size_t index, char *name, size_t name_cap, uint32_t *ggml_type,
+                    uint64_t shape[4], uint32_t *n_dims, size_t *start, size_t *end);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -22,7 +22,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libnative_hip.so")
-SOURCES = ["kernels.hip", "executor.cpp", "residency.cpp"]
+SOURCES = ["kernels.hip", "executor.cpp", "residency.cpp", "gguf.cpp", "llama_host.cpp"]
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # packed-FP32 VALU forms are kept out of every kernel
@@ -117,6 +117,26 @@ def load_library():
         "lnq_admission_requires_eviction": (C.c_int, [sz, sz, sz]),
         "lnq_cache_stats": (None, [psz, psz, psz, psz, psz]),
         "lnq_reset": (None, []),
+        # include/native_hip_llama.h
+        "lnm_last_error": (C.c_char_p, []),
+        "lnm_load": (C.c_int, [C.c_char_p, pvp]),
+        "lnm_load_bytes": (C.c_int, [vp, sz, pvp]),
+        "lnm_free": (None, [vp]),
+        "lnm_info": (C.c_int, [vp, vp]),
+        "lnm_set_products": (C.c_int, [vp, C.c_int, vp, vp]),
+        "lnm_session_new": (C.c_int, [vp, sz, vp, sz, pvp]),
+        "lnm_session_free": (None, [vp]),
+        "lnm_forward": (C.c_int, [vp, vp, sz, vp]),
+        "lnm_generate_greedy": (C.c_int, [vp, vp, sz, sz, vp, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+        "lnm_dequant_row": (C.c_int, [u32, sz, vp, sz, vp]),
+        "lnm_rmsnorm": (C.c_int, [vp, vp, sz, C.c_float]),
+        "lnm_rope": (C.c_int, [vp, sz, sz, sz, C.c_float]),
+        "lnm_softmax": (None, [vp, sz]),
+        "lnm_argmax": (u32, [vp, sz]),
+        "lnm_write_synthetic_llama": (C.c_int, [C.c_char_p, vp]),
+        "lnm_gguf_inspect": (C.c_int, [vp, sz, psz, psz, psz]),
+        "lnm_gguf_tensor": (C.c_int, [vp, sz, sz, C.c_char_p, sz, C.POINTER(u32), C.POINTER(C.c_uint64),
+                                      C.POINTER(u32), psz, psz]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)  # AttributeError if the ABI lost a symbol
@@ -127,7 +147,7 @@ def load_library():
 
 
 def exported_symbols():
-    """Every entry point include/native_hip.h declares (used by the ABI test)."""
+    """Every entry point include/native_hip.h and include/native_hip_llama.h declare (used by the ABI test)."""
     load_library()
     return sorted(_lib._signatures)
 

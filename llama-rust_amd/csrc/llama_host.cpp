@@ -1,0 +1,861 @@
+// Host side of a dense Llama decode over the matrix executor (see include/native_hip_llama.h).
+//
+// Everything here is f32 host arithmetic in the reference's operation order; the only
+// work that leaves the host is the weight products, which go to the executor (or to the
+// caller's function).  Multiplications and additions are never contracted into FMAs, as
+// in the reference's scalar Rust.
+#pragma clang fp contract(off)
+
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <chrono>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <memory>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "../../include/native_hip.h"
+#include "../../include/native_hip_llama.h"
+#include "gguf.h"
+
+namespace {
+
+thread_local std::string t_err;
+int fail(const std::string &m) {
+    t_err = m;
+    return 1;
+}
+
+// ------------------------------------------------------------------ numeric building blocks
+
+float f16_to_f32(uint16_t h) {  // langtax/src/fp16.rs:4-33: exact, subnormals and specials included
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, exp = (h >> 10) & 31u, man = h & 1023u;
+    uint32_t bits;
+    if (exp == 0) {
+        if (man == 0) {
+            bits = sign;
+        } else {  // subnormal: man * 2^-24
+            int e = 0;
+            uint32_t m = man;
+            while (!(m & 1024u)) {
+                m <<= 1;
+                e++;
+            }
+            bits = sign | ((uint32_t)(113 - e) << 23) | ((m & 1023u) << 13);
+        }
+    } else if (exp == 31) {
+        bits = sign | 0x7f800000u | (man << 13);
+    } else {
+        bits = sign | ((exp + 112u) << 23) | (man << 13);
+    }
+    float f;
+    std::memcpy(&f, &bits, 4);
+    return f;
+}
+uint16_t rd16(const uint8_t *p) { return (uint16_t)(p[0] | (p[1] << 8)); }
+uint32_t rd32(const uint8_t *p) { return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24); }
+
+// One packed row -> n_cols floats, bit for bit the value every product of the reference is
+// defined on (langtax/src/quant.rs:7511-7541, 7734-7765, 7884-7950, 8046-8130, 8783-8853).
+bool dequant_row(uint32_t type, size_t n_cols, const uint8_t *row, float *y) {
+    size_t bb = 0, bk = 0;
+    if (!nh::gguf::type_layout(type, &bb, &bk) || n_cols % bk != 0) return false;
+    const size_t nb = n_cols / bk;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *w = row + b * bb;
+        float *o = y + b * bk;
+        switch (type) {
+        case 0: std::memcpy(o, w, 4); break;
+        case 1: o[0] = f16_to_f32(rd16(w)); break;
+        case 8: {
+            const float d = f16_to_f32(rd16(w));
+            for (int j = 0; j < 32; j++) o[j] = (float)(int8_t)w[2 + j] * d;
+            break;
+        }
+        case 2: {
+            const float d = f16_to_f32(rd16(w));
+            for (int j = 0; j < 16; j++) {
+                o[j] = (float)((int)(w[2 + j] & 15) - 8) * d;
+                o[j + 16] = (float)((int)(w[2 + j] >> 4) - 8) * d;
+            }
+            break;
+        }
+        case 6:
+        case 7: {
+            const bool with_min = type == 7;
+            const float d = f16_to_f32(rd16(w)), m = with_min ? f16_to_f32(rd16(w + 2)) : 0.f;
+            const uint32_t qh = rd32(w + (with_min ? 4 : 2));
+            const uint8_t *qs = w + (with_min ? 8 : 6);
+            for (int j = 0; j < 16; j++) {
+                const int lo = (qs[j] & 15) | (int)(((qh >> j) & 1u) << 4);
+                const int hi = (qs[j] >> 4) | (int)(((qh >> (j + 16)) & 1u) << 4);
+                if (with_min) {
+                    const float a = (float)lo * d, c = (float)hi * d;
+                    o[j] = a + m;
+                    o[j + 16] = c + m;
+                } else {
+                    o[j] = (float)(lo - 16) * d;
+                    o[j + 16] = (float)(hi - 16) * d;
+                }
+            }
+            break;
+        }
+        case 12: {
+            const float d = f16_to_f32(rd16(w)), dmin = f16_to_f32(rd16(w + 2));
+            const uint8_t *s = w + 4, *qs = w + 16;
+            for (int pair = 0; pair < 4; pair++) {  // 64 columns: low nibbles, then high nibbles, of 32 bytes
+                for (int half = 0; half < 2; half++) {
+                    const int j = 2 * pair + half;
+                    uint32_t sc, mn;  // langtax/src/quant.rs:8901-8912
+                    if (j < 4) {
+                        sc = s[j] & 63u;
+                        mn = s[j + 4] & 63u;
+                    } else {
+                        sc = (s[j + 4] & 15u) | ((uint32_t)(s[j - 4] >> 6) << 4);
+                        mn = (uint32_t)(s[j + 4] >> 4) | ((uint32_t)(s[j] >> 6) << 4);
+                    }
+                    const float a = d * (float)sc, c = dmin * (float)mn;
+                    for (int l = 0; l < 32; l++) {
+                        const uint32_t q = half ? (uint32_t)(qs[32 * pair + l] >> 4) : (qs[32 * pair + l] & 15u);
+                        const float p = a * (float)q;
+                        o[64 * pair + 32 * half + l] = p - c;
+                    }
+                }
+            }
+            break;
+        }
+        case 14: {
+            const uint8_t *ql = w, *qh = w + 128;
+            const int8_t *sc = reinterpret_cast<const int8_t *>(w + 192);
+            const float d = f16_to_f32(rd16(w + 208));
+            for (int n = 0; n < 2; n++) {  // 128 columns per half
+                for (int l = 0; l < 32; l++) {
+                    const int is = l / 16;
+                    const uint8_t h = qh[32 * n + l];
+                    const int q1 = (int)((ql[64 * n + l] & 15) | ((h & 3) << 4)) - 32;
+                    const int q2 = (int)((ql[64 * n + l + 32] & 15) | (((h >> 2) & 3) << 4)) - 32;
+                    const int q3 = (int)((ql[64 * n + l] >> 4) | (((h >> 4) & 3) << 4)) - 32;
+                    const int q4 = (int)((ql[64 * n + l + 32] >> 4) | (((h >> 6) & 3) << 4)) - 32;
+                    const float d1 = d * (float)sc[8 * n + is], d2 = d * (float)sc[8 * n + is + 2];
+                    const float d3 = d * (float)sc[8 * n + is + 4], d4 = d * (float)sc[8 * n + is + 6];
+                    o[128 * n + l] = d1 * (float)q1;
+                    o[128 * n + l + 32] = d2 * (float)q2;
+                    o[128 * n + l + 64] = d3 * (float)q3;
+                    o[128 * n + l + 96] = d4 * (float)q4;
+                }
+            }
+            break;
+        }
+        default: return false;
+        }
+    }
+    return true;
+}
+
+// langtax/src/decode.rs:11498-11513.  The element count enters as the reference converts it:
+// through u16, anything longer counting as 1.
+void rmsnorm(float *x, const float *w, size_t n, float eps) {
+    float ss = 0.f;
+    for (size_t i = 0; i < n; i++) ss += x[i] * x[i];
+    const float nf = n <= 65535 ? (float)n : 1.f;
+    const float rms = std::sqrt(ss / nf + eps);
+    const float inv = rms > 0.f ? 1.f / rms : 0.f;
+    for (size_t i = 0; i < n; i++) x[i] = x[i] * inv * w[i];
+}
+
+// langtax/src/decode.rs:11578-11602: adjacent pairs, theta multiplied up pair by pair.
+void rope(float *v, size_t len, size_t pos, size_t n_rot, float base) {
+    const size_t n = n_rot < len ? n_rot : len;
+    if (n < 2) return;
+    const float n_rot_f = n_rot <= 65535 ? (float)n_rot : 2.f;
+    float theta = pos <= 65535 ? (float)pos : 65535.f;
+    const float theta_scale = std::pow(base, -2.0f / n_rot_f);
+    for (size_t i = 0; i + 1 < n; i += 2) {
+        const float c = std::cos(theta), s = std::sin(theta);
+        const float x = v[i], y = v[i + 1];
+        v[i] = x * c - y * s;
+        v[i + 1] = x * s + y * c;
+        theta *= theta_scale;
+    }
+}
+
+void softmax(float *x, size_t n) {  // langtax/src/decode.rs:12021-12033
+    float m = -INFINITY;
+    for (size_t i = 0; i < n; i++) m = std::fmax(m, x[i]);
+    float s = 0.f;
+    for (size_t i = 0; i < n; i++) {
+        x[i] = std::exp(x[i] - m);
+        s += x[i];
+    }
+    if (s > 0.f)
+        for (size_t i = 0; i < n; i++) x[i] /= s;
+}
+
+uint32_t argmax(const float *x, size_t n) {  // first maximum wins; langtax/src/decode.rs:12104-12114
+    size_t best_i = 0;
+    float best = -INFINITY;
+    for (size_t i = 0; i < n; i++)
+        if (x[i] > best) {
+            best = x[i];
+            best_i = i;
+        }
+    return (uint32_t)best_i;
+}
+
+// ------------------------------------------------------------------ model
+
+struct Mat {
+    std::string name;
+    uint32_t type = 0;
+    size_t n_rows = 0, n_cols = 0;
+    const uint8_t *bytes = nullptr;
+    size_t nbytes = 0;
+    lnh_matrix *resident = nullptr;
+};
+
+struct Layer {
+    std::vector<float> attn_norm, ffn_norm;
+    Mat wq, wk, wv, wo, gate, up, down;
+};
+
+}  // namespace
+
+struct lnm_model {
+    std::vector<uint8_t> owned;  // lnm_load_bytes
+    void *map = nullptr;         // lnm_load
+    size_t map_len = 0;
+    nh::gguf::File file;
+    lnm_hparams hp{};
+    std::vector<Layer> layers;
+    Mat token_embd, output;
+    std::vector<float> output_norm;
+    int route = LNM_PRODUCTS_RESIDENT;
+    lnm_matmul_fn fn = nullptr;
+    void *user = nullptr;
+    lnh_exec *exec = nullptr;
+
+    ~lnm_model() {
+        auto drop = [](Mat &m) {
+            if (m.resident) lnh_matrix_free(m.resident);
+            m.resident = nullptr;
+        };
+        for (Layer &l : layers)
+            for (Mat *m : {&l.wq, &l.wk, &l.wv, &l.wo, &l.gate, &l.up, &l.down}) drop(*m);
+        drop(token_embd);
+        drop(output);
+        if (exec) lnh_destroy(exec);
+        if (map) munmap(map, map_len);
+    }
+};
+
+struct lnm_session {
+    lnm_model *model = nullptr;
+    size_t kv_block = 16, past = 0;
+    std::vector<uint32_t> table;      // logical block -> physical block
+    std::vector<uint32_t> preset;     // physical ids to hand out, in order (empty: 0, 1, 2, ...)
+    std::vector<float> cache_k, cache_v;
+    std::vector<float> x, residual, q, k, v, attn, attn_proj, gate, up, ffn_out, xn, scores;
+};
+
+namespace {
+
+bool read_f32s(const nh::gguf::File &f, const std::string &name, size_t n, std::vector<float> *out, std::string *err) {
+    const nh::gguf::TensorInfo *t = f.tensor(name);
+    if (!t) return *err = "missing tensor " + name, false;
+    if (t->type != 0 || t->end - t->start != 4 * n) return *err = "tensor " + name + " is not f32[" + std::to_string(n) + "]", false;
+    out->resize(n);
+    std::memcpy(out->data(), f.data + t->start, 4 * n);
+    return true;
+}
+
+bool read_mat(const nh::gguf::File &f, const std::string &name, size_t n_rows, size_t n_cols, Mat *out, std::string *err) {
+    const nh::gguf::TensorInfo *t = f.tensor(name);
+    if (!t) return *err = "missing tensor " + name, false;
+    // ggml order: shape[0] = columns (contiguous), shape[1] = rows
+    if (t->shape.size() != 2 || t->shape[0] != n_cols || t->shape[1] != n_rows)
+        return *err = "tensor " + name + " has the wrong shape", false;
+    out->name = name;
+    out->type = t->type;
+    out->n_rows = n_rows;
+    out->n_cols = n_cols;
+    out->bytes = f.data + t->start;
+    out->nbytes = t->end - t->start;
+    return true;
+}
+
+int finish_load(lnm_model *m) {
+    std::string err;
+    const nh::gguf::File &f = m->file;
+    std::string arch;
+    if (!f.kv_str("general.architecture", &arch)) return fail("missing key general.architecture");
+    if (arch != "llama") return fail("unsupported architecture " + arch);
+    auto need_u32 = [&](const char *field, uint32_t *out) {
+        const std::string key = arch + "." + field;
+        if (!f.kv_u32(key, out)) {
+            err = "missing key " + key;
+            return false;
+        }
+        return true;
+    };
+    lnm_hparams &hp = m->hp;
+    if (!need_u32("block_count", &hp.n_layer) || !need_u32("embedding_length", &hp.n_embd) ||
+        !need_u32("attention.head_count", &hp.n_head) || !need_u32("attention.head_count_kv", &hp.n_head_kv) ||
+        !need_u32("feed_forward_length", &hp.n_ff))
+        return fail(err);
+    if (!hp.n_layer || !hp.n_embd || !hp.n_head || !hp.n_head_kv || !hp.n_ff) return fail("zero hyper-parameter");
+    if (hp.n_head % hp.n_head_kv != 0 || hp.n_embd % hp.n_head != 0) return fail("head counts do not divide");
+    hp.head_dim = hp.n_embd / hp.n_head;
+    if (!f.kv_u32(arch + ".rope.dimension_count", &hp.n_rot)) hp.n_rot = hp.head_dim;  // decode.rs:7461-7475
+    if (hp.n_rot == 0) return fail("zero rope.dimension_count");
+    if (!f.kv_f32(arch + ".rope.freq_base", &hp.rope_base)) hp.rope_base = 10000.f;                  // decode.rs:2053
+    if (!f.kv_f32(arch + ".attention.layer_norm_rms_epsilon", &hp.rms_eps)) hp.rms_eps = 1e-5f;      // decode.rs:1958
+    const nh::gguf::TensorInfo *emb = f.tensor("token_embd.weight");
+    if (!emb || emb->shape.size() != 2 || emb->shape[0] != hp.n_embd) return fail("missing or misshapen token_embd.weight");
+    hp.n_vocab = (uint32_t)emb->shape[1];
+    if (!read_mat(f, "token_embd.weight", hp.n_vocab, hp.n_embd, &m->token_embd, &err)) return fail(err);
+    if (!read_f32s(f, "output_norm.weight", hp.n_embd, &m->output_norm, &err)) return fail(err);
+    if (f.tensor("output.weight")) {
+        if (!read_mat(f, "output.weight", hp.n_vocab, hp.n_embd, &m->output, &err)) return fail(err);
+    } else {
+        m->output = m->token_embd;  // tied head (decode.rs:2069-2072)
+    }
+    const size_t qw = (size_t)hp.n_head * hp.head_dim, kvw = (size_t)hp.n_head_kv * hp.head_dim;
+    m->layers.resize(hp.n_layer);
+    for (uint32_t i = 0; i < hp.n_layer; i++) {
+        Layer &l = m->layers[i];
+        const std::string p = "blk." + std::to_string(i) + ".";
+        if (!read_f32s(f, p + "attn_norm.weight", hp.n_embd, &l.attn_norm, &err) ||
+            !read_f32s(f, p + "ffn_norm.weight", hp.n_embd, &l.ffn_norm, &err) ||
+            !read_mat(f, p + "attn_q.weight", qw, hp.n_embd, &l.wq, &err) ||
+            !read_mat(f, p + "attn_k.weight", kvw, hp.n_embd, &l.wk, &err) ||
+            !read_mat(f, p + "attn_v.weight", kvw, hp.n_embd, &l.wv, &err) ||
+            !read_mat(f, p + "attn_output.weight", hp.n_embd, qw, &l.wo, &err) ||
+            !read_mat(f, p + "ffn_gate.weight", hp.n_ff, hp.n_embd, &l.gate, &err) ||
+            !read_mat(f, p + "ffn_up.weight", hp.n_ff, hp.n_embd, &l.up, &err) ||
+            !read_mat(f, p + "ffn_down.weight", hp.n_embd, hp.n_ff, &l.down, &err))
+            return fail(err);
+    }
+    hp.block_type = m->layers[0].wq.type;
+    hp.embd_type = m->token_embd.type;
+    hp.output_type = m->output.type;
+    return 0;
+}
+
+// One weight product, by the model's route.
+int product(lnm_model *m, Mat &w, size_t n, const float *x, float *y) {
+    const size_t x_len = n * w.n_cols, y_len = n * w.n_rows;
+    switch (m->route) {
+    case LNM_PRODUCTS_CALLBACK:
+        if (!m->fn) return fail("no product function set");
+        if (m->fn(m->user, w.type, w.n_rows, w.n_cols, n, w.bytes, w.nbytes, x, y) != 0)
+            return fail("product function failed for " + w.name);
+        return 0;
+    case LNM_PRODUCTS_DISPATCH: {
+        const int rc = n == 1 ? lnq_gemv(w.type, w.n_cols, w.bytes, w.nbytes, x, x_len, y, y_len)
+                              : lnq_gemm(w.type, w.n_cols, n, w.bytes, w.nbytes, x, x_len, y, y_len);
+        return rc == 0 ? 0 : fail(std::string(lnq_last_error()) + " (" + w.name + ")");
+    }
+    default: {
+        if (!m->exec && lnh_create(0, &m->exec) != 0) return fail(std::string("executor: ") + lnh_thread_error());
+        if (!w.resident &&
+            lnh_upload_packed(m->exec, w.type, w.n_rows, w.n_cols, w.bytes, w.nbytes, &w.resident) != 0)
+            return fail(std::string(lnh_last_error(m->exec)) + " (" + w.name + ")");
+        if (lnh_gemm(m->exec, w.resident, n, x, x_len, y, y_len) != 0)
+            return fail(std::string(lnh_last_error(m->exec)) + " (" + w.name + ")");
+        return 0;
+    }
+    }
+}
+
+// langtax/src/kv_page.rs:410-438, paged branch.
+size_t kv_offset(const lnm_session *s, size_t layer, size_t head, size_t t) {
+    const lnm_hparams &hp = s->model->hp;
+    const size_t bs = s->kv_block, b = s->table[t / bs];
+    return ((((size_t)b * hp.n_layer + layer) * hp.n_head_kv + head) * bs + t % bs) * hp.head_dim;
+}
+
+int ensure_blocks(lnm_session *s, size_t positions) {
+    const lnm_hparams &hp = s->model->hp;
+    const size_t need = (positions + s->kv_block - 1) / s->kv_block;
+    while (s->table.size() < need) {
+        uint32_t id = (uint32_t)s->table.size();
+        if (!s->preset.empty()) {
+            if (s->table.size() >= s->preset.size()) return fail("sequence outgrew the given block ids");
+            id = s->preset[s->table.size()];
+        }
+        s->table.push_back(id);
+        const size_t stride = (size_t)hp.n_layer * hp.n_head_kv * s->kv_block * hp.head_dim;
+        const size_t floats = ((size_t)id + 1) * stride;
+        if (s->cache_k.size() < floats) {
+            s->cache_k.resize(floats, 0.f);
+            s->cache_v.resize(floats, 0.f);
+        }
+    }
+    return 0;
+}
+
+// langtax/src/decode.rs:2710-3099, dense llama branch, LogitsKind::Last.
+int forward(lnm_session *s, const uint32_t *tokens, size_t n, float *logits) {
+    lnm_model *m = s->model;
+    const lnm_hparams &hp = m->hp;
+    if (n == 0) return fail("empty batch");
+    const size_t d = hp.n_embd, hd = hp.head_dim, qw = (size_t)hp.n_head * hd, kvw = (size_t)hp.n_head_kv * hd;
+    const size_t gqa = hp.n_head / hp.n_head_kv;
+    if (ensure_blocks(s, s->past + n) != 0) return 1;
+    s->x.resize(n * d);
+    const size_t emb_row = m->token_embd.nbytes / m->token_embd.n_rows;
+    for (size_t t = 0; t < n; t++) {
+        if (tokens[t] >= hp.n_vocab) return fail("token id out of range");
+        if (!dequant_row(m->token_embd.type, d, m->token_embd.bytes + (size_t)tokens[t] * emb_row, &s->x[t * d]))
+            return fail("cannot dequantize token_embd.weight");
+    }
+    s->q.resize(n * qw);
+    s->k.resize(n * kvw);
+    s->v.resize(n * kvw);
+    s->attn.resize(n * qw);
+    s->attn_proj.resize(n * d);
+    s->gate.resize(n * hp.n_ff);
+    s->up.resize(n * hp.n_ff);
+    s->ffn_out.resize(n * d);
+    const float hd_f = hd <= 65535 ? (float)hd : 1.f;
+    const float root = std::sqrt(hd_f);
+    const float score_scale = root > 0.f ? 1.f / root : 0.f;
+
+    for (size_t li = 0; li < hp.n_layer; li++) {
+        Layer &l = m->layers[li];
+        s->residual = s->x;
+        for (size_t t = 0; t < n; t++) rmsnorm(&s->x[t * d], l.attn_norm.data(), d, hp.rms_eps);
+        if (product(m, l.wq, n, s->x.data(), s->q.data()) || product(m, l.wk, n, s->x.data(), s->k.data()) ||
+            product(m, l.wv, n, s->x.data(), s->v.data()))
+            return 1;
+        for (size_t t = 0; t < n; t++) {  // rotate and store K, store V
+            const size_t p = s->past + t;
+            float *kt = &s->k[t * kvw];
+            for (size_t h = 0; h < hp.n_head_kv; h++) {
+                rope(kt + h * hd, hd, p, hp.n_rot, hp.rope_base);
+                std::memcpy(&s->cache_k[kv_offset(s, li, h, p)], kt + h * hd, hd * sizeof(float));
+                std::memcpy(&s->cache_v[kv_offset(s, li, h, p)], &s->v[t * kvw + h * hd], hd * sizeof(float));
+            }
+        }
+        for (size_t t = 0; t < n; t++) {  // decode.rs:11126-11197
+            const size_t p = s->past + t, seq = p + 1;
+            float *qt = &s->q[t * qw];
+            s->scores.resize(seq);
+            for (size_t hq = 0; hq < hp.n_head; hq++) {
+                float *qv = qt + hq * hd;
+                rope(qv, hd, p, hp.n_rot, hp.rope_base);
+                const size_t hkv = hq / gqa;
+                for (size_t u = 0; u < seq; u++) {
+                    const float *kv = &s->cache_k[kv_offset(s, li, hkv, u)];
+                    float dot = 0.f;
+                    for (size_t i = 0; i < hd; i++) dot += qv[i] * kv[i];
+                    s->scores[u] = dot * score_scale;
+                }
+                softmax(s->scores.data(), seq);
+                float *dst = &s->attn[t * qw + hq * hd];
+                for (size_t i = 0; i < hd; i++) dst[i] = 0.f;
+                for (size_t u = 0; u < seq; u++) {
+                    const float *vv = &s->cache_v[kv_offset(s, li, hkv, u)];
+                    const float st = s->scores[u];
+                    for (size_t i = 0; i < hd; i++) dst[i] += st * vv[i];
+                }
+            }
+        }
+        if (product(m, l.wo, n, s->attn.data(), s->attn_proj.data())) return 1;
+        for (size_t i = 0; i < n * d; i++) s->x[i] = s->attn_proj[i] + s->residual[i];
+        s->residual = s->x;
+        for (size_t t = 0; t < n; t++) rmsnorm(&s->x[t * d], l.ffn_norm.data(), d, hp.rms_eps);
+        if (product(m, l.gate, n, s->x.data(), s->gate.data()) || product(m, l.up, n, s->x.data(), s->up.data()))
+            return 1;
+        for (size_t i = 0; i < n * hp.n_ff; i++) {  // SiLU(gate) * up, decode.rs:11826-11830 and 2981-2984
+            const float g = s->gate[i];
+            s->gate[i] = g / (1.f + std::exp(-g));
+            s->gate[i] *= s->up[i];
+        }
+        if (product(m, l.down, n, s->gate.data(), s->ffn_out.data())) return 1;
+        for (size_t i = 0; i < n * d; i++) s->x[i] = s->ffn_out[i] + s->residual[i];
+    }
+    s->xn.assign(s->x.begin() + (n - 1) * d, s->x.begin() + n * d);
+    rmsnorm(s->xn.data(), m->output_norm.data(), d, hp.rms_eps);
+    if (product(m, m->output, 1, s->xn.data(), logits)) return 1;
+    s->past += n;
+    return 0;
+}
+
+// ------------------------------------------------------------------ synthetic model
+
+uint64_t splitmix(uint64_t &st) {  // langtax/src/sample.rs SplitMix64
+    st += 0x9e3779b97f4a7c15ull;
+    uint64_t z = st;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+}
+struct Rng {
+    uint64_t st;
+    uint64_t next() { return splitmix(st); }
+    float uniform() { return (float)(next() >> 40) * (1.0f / 16777216.0f); }  // top 24 bits -> [0, 1)
+    float normal() {
+        const float u1 = 1.0f - uniform(), u2 = uniform();
+        return std::sqrt(-2.0f * std::log(u1)) * std::cos(6.28318530717958647692f * u2);
+    }
+};
+
+uint16_t f32_to_f16(float f) {  // round to nearest even; enough for scales this generator draws
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    const int32_t e = (int32_t)((x >> 23) & 255u) - 127 + 15;
+    uint32_t man = x & 0x7fffffu;
+    if (e >= 31) return (uint16_t)(sign | 0x7c00u);
+    if (e <= 0) {
+        if (e < -10) return (uint16_t)sign;
+        man |= 0x800000u;
+        const int shift = 14 - e;
+        uint32_t h = man >> shift;
+        const uint32_t rem = man & ((1u << shift) - 1), halfway = 1u << (shift - 1);
+        if (rem > halfway || (rem == halfway && (h & 1u))) h++;
+        return (uint16_t)(sign | h);
+    }
+    uint32_t h = ((uint32_t)e << 10) | (man >> 13);
+    const uint32_t rem = man & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) h++;
+    return (uint16_t)(sign | h);
+}
+void wr16(uint8_t *p, uint16_t v) {
+    p[0] = (uint8_t)v;
+    p[1] = (uint8_t)(v >> 8);
+}
+
+// Random packed rows whose dequantized values have mean 0 and standard deviation sigma.
+void random_rows(uint32_t type, size_t n_cols, size_t n_rows, float sigma, uint64_t seed, uint8_t *dst) {
+    size_t bb = 0, bk = 0;
+    nh::gguf::type_layout(type, &bb, &bk);
+    const size_t row_bytes = n_cols / bk * bb, chunk = 64;  // rows per independent random stream
+    const size_t n_chunks = (n_rows + chunk - 1) / chunk;
+    unsigned hw = std::thread::hardware_concurrency();
+    const size_t n_threads = hw < 1 ? 1 : (hw > 16 ? 16 : hw);
+    auto work = [&](size_t tid) {
+        for (size_t c = tid; c < n_chunks; c += n_threads) {
+            Rng r{seed ^ (0x51ed270b0a1f3c5dull * (c + 1))};
+            const size_t r0 = c * chunk, r1 = r0 + chunk < n_rows ? r0 + chunk : n_rows;
+            for (uint8_t *w = dst + r0 * row_bytes; w < dst + r1 * row_bytes; w += bb) {
+                switch (type) {
+                case 0: {
+                    const float v = sigma * r.normal();
+                    std::memcpy(w, &v, 4);
+                    break;
+                }
+                case 1: wr16(w, f32_to_f16(sigma * r.normal())); break;
+                case 8:  // codes uniform in [-127, 127]: rms 73.3
+                    wr16(w, f32_to_f16(std::fabs(r.normal()) * sigma / 73.3f));
+                    for (int j = 0; j < 32; j++) w[2 + j] = (uint8_t)(int8_t)((int)(r.next() % 255u) - 127);
+                    break;
+                case 2:  // nibble - 8: rms 4.64
+                    wr16(w, f32_to_f16(r.normal() * sigma / 4.64f));
+                    for (int j = 0; j < 16; j += 8) {
+                        const uint64_t v = r.next();
+                        std::memcpy(w + 2 + j, &v, 8);
+                    }
+                    break;
+                case 6:  // code - 16: rms 9.25
+                    wr16(w, f32_to_f16(r.normal() * sigma / 9.25f));
+                    for (int j = 0; j < 20; j += 4) {
+                        const uint32_t v = (uint32_t)r.next();
+                        std::memcpy(w + 2 + j, &v, 4);
+                    }
+                    break;
+                case 7: {  // code * d + m with m = -15.5 d: standard deviation 9.23 |d|
+                    const float d = r.normal() * sigma / 9.23f;
+                    wr16(w, f32_to_f16(d));
+                    wr16(w + 2, f32_to_f16(-15.5f * d));
+                    for (int j = 0; j < 20; j += 4) {
+                        const uint32_t v = (uint32_t)r.next();
+                        std::memcpy(w + 4 + j, &v, 4);
+                    }
+                    break;
+                }
+                case 12: {  // d sc q - dmin m, all codes uniform: mean 0 for dmin = 7.5 d, deviation 258 d
+                    const float d = std::fabs(r.normal()) * sigma / 258.f;
+                    wr16(w, f32_to_f16(d));
+                    wr16(w + 2, f32_to_f16(7.5f * d));
+                    for (int j = 0; j < 140; j += 4) {
+                        const uint32_t v = (uint32_t)r.next();
+                        std::memcpy(w + 4 + j, &v, 4);
+                    }
+                    break;
+                }
+                default: {  // Q6_K: d sc (q - 32), sc uniform in [-32, 31]: deviation 341 d
+                    for (int j = 0; j < 192; j += 8) {
+                        const uint64_t v = r.next();
+                        std::memcpy(w + j, &v, 8);
+                    }
+                    for (int j = 0; j < 16; j++) w[192 + j] = (uint8_t)(int8_t)((int)(r.next() & 63u) - 32);
+                    wr16(w + 208, f32_to_f16(std::fabs(r.normal()) * sigma / 341.f));
+                    break;
+                }
+                }
+            }
+        }
+    };
+    std::vector<std::thread> pool;
+    for (size_t t = 1; t < n_threads; t++) pool.emplace_back(work, t);
+    work(0);
+    for (auto &t : pool) t.join();
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------ C ABI
+
+extern "C" {
+
+const char *lnm_last_error(void) { return t_err.c_str(); }
+
+int lnm_load_bytes(const uint8_t *bytes, size_t len, lnm_model **out) {
+    if (!bytes || !out) return fail("null argument");
+    std::unique_ptr<lnm_model> m(new lnm_model);
+    m->owned.assign(bytes, bytes + len);
+    std::string err;
+    if (!nh::gguf::parse(m->owned.data(), m->owned.size(), &m->file, &err)) return fail("gguf: " + err);
+    if (finish_load(m.get()) != 0) return 1;
+    *out = m.release();
+    return 0;
+}
+
+int lnm_load(const char *path, lnm_model **out) {
+    if (!path || !out) return fail("null argument");
+    const int fd = open(path, O_RDONLY);
+    if (fd < 0) return fail(std::string("cannot open ") + path);
+    struct stat st;
+    if (fstat(fd, &st) != 0 || st.st_size <= 0) {
+        close(fd);
+        return fail(std::string("cannot stat ") + path);
+    }
+    void *p = mmap(nullptr, (size_t)st.st_size, PROT_READ, MAP_PRIVATE, fd, 0);
+    close(fd);
+    if (p == MAP_FAILED) return fail(std::string("cannot map ") + path);
+    std::unique_ptr<lnm_model> m(new lnm_model);
+    m->map = p;
+    m->map_len = (size_t)st.st_size;
+    std::string err;
+    if (!nh::gguf::parse(static_cast<const uint8_t *>(p), m->map_len, &m->file, &err)) return fail("gguf: " + err);
+    if (finish_load(m.get()) != 0) return 1;
+    *out = m.release();
+    return 0;
+}
+
+void lnm_free(lnm_model *model) { delete model; }
+
+int lnm_info(const lnm_model *model, lnm_hparams *out) {
+    if (!model || !out) return fail("null argument");
+    *out = model->hp;
+    return 0;
+}
+
+int lnm_set_products(lnm_model *model, int route, lnm_matmul_fn fn, void *user) {
+    if (!model) return fail("null argument");
+    if (route < LNM_PRODUCTS_RESIDENT || route > LNM_PRODUCTS_CALLBACK) return fail("unknown product route");
+    if (route == LNM_PRODUCTS_CALLBACK && !fn) return fail("callback route without a function");
+    model->route = route;
+    model->fn = fn;
+    model->user = user;
+    return 0;
+}
+
+int lnm_session_new(lnm_model *model, size_t kv_block, const uint32_t *block_ids, size_t n_block_ids,
+                    lnm_session **out) {
+    if (!model || !out) return fail("null argument");
+    if (kv_block == 0) return fail("zero K/V block size");
+    std::unique_ptr<lnm_session> s(new lnm_session);
+    s->model = model;
+    s->kv_block = kv_block;
+    if (block_ids) {
+        std::vector<bool> seen(n_block_ids, false);
+        for (size_t i = 0; i < n_block_ids; i++) {
+            if (block_ids[i] >= n_block_ids || seen[block_ids[i]]) return fail("block ids are not a permutation");
+            seen[block_ids[i]] = true;
+        }
+        s->preset.assign(block_ids, block_ids + n_block_ids);
+    }
+    *out = s.release();
+    return 0;
+}
+
+void lnm_session_free(lnm_session *session) { delete session; }
+
+int lnm_forward(lnm_session *session, const uint32_t *tokens, size_t n, float *logits) {
+    if (!session || !tokens || !logits) return fail("null argument");
+    return forward(session, tokens, n, logits);
+}
+
+int lnm_generate_greedy(lnm_session *session, const uint32_t *prompt, size_t n_prompt, size_t n_new,
+                        uint32_t *out, double *prefill_seconds, double *decode_seconds) {
+    if (!session || !prompt || !out) return fail("null argument");
+    if (n_prompt == 0 || n_new == 0) return fail("empty prompt or nothing to generate");
+    std::vector<float> logits(session->model->hp.n_vocab);
+    using clock = std::chrono::steady_clock;
+    const auto t0 = clock::now();
+    if (forward(session, prompt, n_prompt, logits.data()) != 0) return 1;
+    out[0] = argmax(logits.data(), logits.size());
+    const auto t1 = clock::now();
+    for (size_t i = 1; i < n_new; i++) {
+        if (forward(session, &out[i - 1], 1, logits.data()) != 0) return 1;
+        out[i] = argmax(logits.data(), logits.size());
+    }
+    const auto t2 = clock::now();
+    if (prefill_seconds) *prefill_seconds = std::chrono::duration<double>(t1 - t0).count();
+    if (decode_seconds) *decode_seconds = std::chrono::duration<double>(t2 - t1).count();
+    return 0;
+}
+
+int lnm_dequant_row(uint32_t ggml_type, size_t n_cols, const uint8_t *row, size_t row_len, float *y) {
+    size_t bb = 0, bk = 0;
+    if (!row || !y) return fail("null argument");
+    if (!nh::gguf::type_layout(ggml_type, &bb, &bk)) return fail("unsupported ggml type " + std::to_string(ggml_type));
+    if (n_cols % bk != 0 || row_len != n_cols / bk * bb) return fail("row length does not match the column count");
+    return dequant_row(ggml_type, n_cols, row, y) ? 0 : fail("cannot dequantize");
+}
+
+int lnm_rmsnorm(float *x, const float *w, size_t n, float eps) {
+    if (!x || !w) return fail("null argument");
+    rmsnorm(x, w, n, eps);
+    return 0;
+}
+
+int lnm_rope(float *head, size_t head_len, size_t pos, size_t n_rot, float base) {
+    if (!head) return fail("null argument");
+    rope(head, head_len, pos, n_rot, base);
+    return 0;
+}
+
+void lnm_softmax(float *x, size_t n) {
+    if (x) softmax(x, n);
+}
+
+uint32_t lnm_argmax(const float *x, size_t n) { return x ? argmax(x, n) : 0; }
+
+int lnm_write_synthetic_llama(const char *path, const lnm_synth_spec *sp) {
+    if (!path || !sp) return fail("null argument");
+    if (!sp->n_layer || !sp->n_embd || !sp->n_head || !sp->n_head_kv || !sp->n_ff || !sp->n_vocab)
+        return fail("zero hyper-parameter");
+    if (sp->n_head % sp->n_head_kv != 0 || sp->n_embd % sp->n_head != 0) return fail("head counts do not divide");
+    size_t bb, bk;
+    for (uint32_t t : {sp->block_type, sp->embd_type, sp->output_type}) {
+        if (!nh::gguf::type_layout(t, &bb, &bk)) return fail("unsupported ggml type " + std::to_string(t));
+        if (sp->n_embd % bk != 0 || sp->n_ff % bk != 0) return fail("row lengths are not whole blocks");
+    }
+    using nh::gguf::Kv;
+    const size_t d = sp->n_embd, hd = d / sp->n_head, qw = (size_t)sp->n_head * hd, kvw = (size_t)sp->n_head_kv * hd;
+    std::vector<std::pair<std::string, Kv>> kv = {
+        {"general.alignment", Kv::u32(32)},
+        {"general.name", Kv::str("native-hip synthetic llama")},
+        {"general.architecture", Kv::str("llama")},
+        {"llama.block_count", Kv::u32(sp->n_layer)},
+        {"llama.context_length", Kv::u32(8192)},
+        {"llama.embedding_length", Kv::u32(sp->n_embd)},
+        {"llama.feed_forward_length", Kv::u32(sp->n_ff)},
+        {"llama.attention.head_count", Kv::u32(sp->n_head)},
+        {"llama.attention.head_count_kv", Kv::u32(sp->n_head_kv)},
+        {"llama.rope.dimension_count", Kv::u32((uint32_t)hd)},
+        {"llama.rope.freq_base", Kv::f32(sp->rope_base)},
+        {"llama.attention.layer_norm_rms_epsilon", Kv::f32(sp->rms_eps)},
+        {"llama.vocab_size", Kv::u32(sp->n_vocab)},
+    };
+    std::vector<nh::gguf::TensorWrite> tensors;
+    uint64_t serial = 0;
+    const uint64_t seed = sp->seed;
+    const float sigma = sp->weight_std;
+    auto mat = [&](const std::string &name, uint32_t type, size_t n_rows, size_t n_cols) {
+        nh::gguf::TensorWrite t;
+        t.name = name;
+        t.type = type;
+        t.shape = {n_cols, n_rows};
+        size_t b = 0, k = 0;
+        nh::gguf::type_layout(type, &b, &k);
+        t.nbytes = n_rows * (n_cols / k * b);
+        uint64_t st = seed + 0x9e3779b97f4a7c15ull * ++serial;
+        const uint64_t tensor_seed = splitmix(st);
+        t.fill = [=](uint8_t *dst) { random_rows(type, n_cols, n_rows, sigma, tensor_seed, dst); };
+        tensors.push_back(std::move(t));
+    };
+    auto norm = [&](const std::string &name) {
+        nh::gguf::TensorWrite t;
+        t.name = name;
+        t.type = 0;
+        t.shape = {d};
+        t.nbytes = 4 * d;
+        uint64_t st = seed + 0x9e3779b97f4a7c15ull * ++serial;
+        const uint64_t tensor_seed = splitmix(st);
+        t.fill = [=](uint8_t *dst) {
+            Rng r{tensor_seed};
+            for (size_t i = 0; i < d; i++) {
+                const float v = 1.0f + 0.05f * r.normal();
+                std::memcpy(dst + 4 * i, &v, 4);
+            }
+        };
+        tensors.push_back(std::move(t));
+    };
+    mat("token_embd.weight", sp->embd_type, sp->n_vocab, d);
+    for (uint32_t i = 0; i < sp->n_layer; i++) {
+        const std::string p = "blk." + std::to_string(i) + ".";
+        norm(p + "attn_norm.weight");
+        mat(p + "attn_q.weight", sp->block_type, qw, d);
+        mat(p + "attn_k.weight", sp->block_type, kvw, d);
+        mat(p + "attn_v.weight", sp->block_type, kvw, d);
+        mat(p + "attn_output.weight", sp->block_type, d, qw);
+        norm(p + "ffn_norm.weight");
+        mat(p + "ffn_gate.weight", sp->block_type, sp->n_ff, d);
+        mat(p + "ffn_up.weight", sp->block_type, sp->n_ff, d);
+        mat(p + "ffn_down.weight", sp->block_type, d, sp->n_ff);
+    }
+    norm("output_norm.weight");
+    mat("output.weight", sp->output_type, sp->n_vocab, d);
+    FILE *f = std::fopen(path, "wb");
+    if (!f) return fail(std::string("cannot create ") + path);
+    std::string err;
+    const bool ok = nh::gguf::write(f, kv, tensors, &err);
+    if (std::fclose(f) != 0 && ok) return fail("write failed");
+    return ok ? 0 : fail("gguf: " + err);
+}
+
+int lnm_gguf_inspect(const uint8_t *bytes, size_t len, size_t *n_tensors, size_t *n_kv, size_t *alignment) {
+    if (!bytes) return fail("null argument");
+    nh::gguf::File f;
+    std::string err;
+    if (!nh::gguf::parse(bytes, len, &f, &err)) return fail("gguf: " + err);
+    if (n_tensors) *n_tensors = f.tensors.size();
+    if (n_kv) *n_kv = f.kv.size();
+    if (alignment) *alignment = f.alignment;
+    return 0;
+}
+
+int lnm_gguf_tensor(const uint8_t *bytes, size_t len, size_t index, char *name, size_t name_cap, uint32_t *ggml_type,
+                    uint64_t shape[4], uint32_t *n_dims, size_t *start, size_t *end) {
+    if (!bytes) return fail("null argument");
+    nh::gguf::File f;
+    std::string err;
+    if (!nh::gguf::parse(bytes, len, &f, &err)) return fail("gguf: " + err);
+    if (index >= f.tensors.size()) return fail("tensor index out of range");
+    const nh::gguf::TensorInfo &t = f.tensors[index];
+    if (name && name_cap) {
+        const size_t k = t.name.size() < name_cap - 1 ? t.name.size() : name_cap - 1;
+        std::memcpy(name, t.name.data(), k);
+        name[k] = 0;
+    }
+    if (ggml_type) *ggml_type = t.type;
+    if (n_dims) *n_dims = (uint32_t)t.shape.size();
+    if (shape)
+        for (size_t i = 0; i < 4; i++) shape[i] = i < t.shape.size() ? t.shape[i] : 1;
+    if (start) *start = t.start;
+    if (end) *end = t.end;
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,199 @@
+"""Host side of a dense Llama decode over the matrix executor, seen from Python.
+
+A ctypes view of include/native_hip_llama.h: GGUF model load, the forward pass
+of langtax/src/decode.rs:2710-3099 (dense llama branch) with a paged K/V cache,
+greedy generation, and the generator of random GGUF models the tests and the
+benchmark use.  The weight products run on the GPU (`RESIDENT`, `DISPATCH`) or
+in a function of the caller (`CALLBACK`, which is how the tests put their CPU
+checker underneath the same host code).
+"""
+import ctypes as C
+import importlib
+
+import numpy as np
+
+_pkg = importlib.import_module(__name__.rsplit(".", 1)[0])
+
+RESIDENT, DISPATCH, CALLBACK = 0, 1, 2
+
+MATMUL_FN = C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_uint32, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p,
+                        C.c_size_t, C.c_void_p, C.c_void_p)
+
+
+class HParams(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("n_layer", "n_embd", "n_head", "n_head_kv", "n_ff", "n_vocab",
+                                            "head_dim", "n_rot")] + \
+               [("rope_base", C.c_float), ("rms_eps", C.c_float)] + \
+               [(n, C.c_uint32) for n in ("block_type", "embd_type", "output_type")]
+
+
+class SynthSpec(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("n_layer", "n_embd", "n_head", "n_head_kv", "n_ff", "n_vocab",
+                                            "block_type", "embd_type", "output_type")] + \
+               [("rope_base", C.c_float), ("rms_eps", C.c_float), ("weight_std", C.c_float), ("seed", C.c_uint64)]
+
+
+class LlamaError(RuntimeError):
+    pass
+
+
+def _check(rc):
+    if rc != 0:
+        raise LlamaError(_pkg.load_library().lnm_last_error().decode())
+
+
+def write_synthetic_llama(path, *, n_layer, n_embd, n_head, n_head_kv, n_ff, n_vocab, block_type=_pkg.Q4_K,
+                          embd_type=_pkg.Q4_K, output_type=_pkg.Q6_K, rope_base=5e5, rms_eps=1e-5,
+                          weight_std=0.02, seed=0):
+    spec = SynthSpec(n_layer, n_embd, n_head, n_head_kv, n_ff, n_vocab, block_type, embd_type, output_type,
+                     rope_base, rms_eps, weight_std, seed)
+    _check(_pkg.load_library().lnm_write_synthetic_llama(str(path).encode(), C.byref(spec)))
+
+
+def gguf_tensors(blob):
+    """[(name, ggml_type, shape, start, end)] of a GGUF blob (bytes or uint8 array)."""
+    lib = _pkg.load_library()
+    a = np.frombuffer(blob, dtype=np.uint8) if not isinstance(blob, np.ndarray) else blob
+    n_t, n_kv, al = C.c_size_t(), C.c_size_t(), C.c_size_t()
+    _check(lib.lnm_gguf_inspect(a.ctypes.data, a.size, C.byref(n_t), C.byref(n_kv), C.byref(al)))
+    out = []
+    for i in range(n_t.value):
+        name = C.create_string_buffer(256)
+        ty, nd, st, en = C.c_uint32(), C.c_uint32(), C.c_size_t(), C.c_size_t()
+        shape = (C.c_uint64 * 4)()
+        _check(lib.lnm_gguf_tensor(a.ctypes.data, a.size, i, name, 256, C.byref(ty), shape, C.byref(nd),
+                                   C.byref(st), C.byref(en)))
+        out.append((name.value.decode(), ty.value, tuple(shape[:nd.value]), st.value, en.value))
+    return out
+
+
+def gguf_inspect(blob):
+    lib = _pkg.load_library()
+    a = np.frombuffer(blob, dtype=np.uint8) if not isinstance(blob, np.ndarray) else blob
+    n_t, n_kv, al = C.c_size_t(), C.c_size_t(), C.c_size_t()
+    _check(lib.lnm_gguf_inspect(a.ctypes.data, a.size, C.byref(n_t), C.byref(n_kv), C.byref(al)))
+    return n_t.value, n_kv.value, al.value
+
+
+def dequant_row(ggml_type, n_cols, row):
+    row = np.ascontiguousarray(row, dtype=np.uint8)
+    y = np.empty(n_cols, dtype=np.float32)
+    _check(_pkg.load_library().lnm_dequant_row(ggml_type, n_cols, row.ctypes.data, row.size, y.ctypes.data))
+    return y
+
+
+def rmsnorm(x, w, eps):
+    x = np.array(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    _check(_pkg.load_library().lnm_rmsnorm(x.ctypes.data, w.ctypes.data, x.size, eps))
+    return x
+
+
+def rope(head, pos, n_rot, base):
+    v = np.array(head, dtype=np.float32)
+    _check(_pkg.load_library().lnm_rope(v.ctypes.data, v.size, pos, n_rot, base))
+    return v
+
+
+def softmax(x):
+    v = np.array(x, dtype=np.float32)
+    _pkg.load_library().lnm_softmax(v.ctypes.data, v.size)
+    return v
+
+
+def argmax(x):
+    v = np.ascontiguousarray(x, dtype=np.float32)
+    return _pkg.load_library().lnm_argmax(v.ctypes.data, v.size)
+
+
+class Llama:
+    """A loaded model; `products` picks the route of the weight products."""
+
+    def __init__(self, path=None, blob=None, products=RESIDENT, matmul=None):
+        lib = _pkg.load_library()
+        h = C.c_void_p()
+        if path is not None:
+            _check(lib.lnm_load(str(path).encode(), C.byref(h)))
+        else:
+            a = np.frombuffer(blob, dtype=np.uint8) if not isinstance(blob, np.ndarray) else blob
+            _check(lib.lnm_load_bytes(a.ctypes.data, a.size, C.byref(h)))
+        self._h = h
+        self._cb = None
+        hp = HParams()
+        _check(lib.lnm_info(h, C.byref(hp)))
+        self.hparams = hp
+        self.set_products(products, matmul)
+
+    def set_products(self, route, matmul=None):
+        """matmul(ggml_type, n_rows, n_cols, n_tokens, w: uint8[w_len], x: f32[n_tokens, n_cols]) -> y."""
+        lib = _pkg.load_library()
+        cb = None
+        if route == CALLBACK:
+            def thunk(_user, ty, n_rows, n_cols, n_tokens, w, w_len, x, y):
+                try:
+                    wa = np.ctypeslib.as_array(C.cast(w, C.POINTER(C.c_uint8)), shape=(w_len,))
+                    xa = np.ctypeslib.as_array(C.cast(x, C.POINTER(C.c_float)), shape=(n_tokens, n_cols))
+                    ya = np.ctypeslib.as_array(C.cast(y, C.POINTER(C.c_float)), shape=(n_tokens, n_rows))
+                    ya[...] = matmul(ty, n_rows, n_cols, n_tokens, wa, xa)
+                    return 0
+                except Exception:  # the C side reports the failure
+                    import traceback
+                    traceback.print_exc()
+                    return 1
+            cb = MATMUL_FN(thunk)
+        _check(lib.lnm_set_products(self._h, route, C.cast(cb, C.c_void_p) if cb else None, None))
+        self._cb = cb  # keep the thunk alive
+
+    def session(self, kv_block=16, block_ids=None):
+        return Session(self, kv_block, block_ids)
+
+    def close(self):
+        if self._h:
+            _pkg.load_library().lnm_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Session:
+    def __init__(self, model, kv_block=16, block_ids=None):
+        lib = _pkg.load_library()
+        self.model = model
+        h = C.c_void_p()
+        if block_ids is None:
+            _check(lib.lnm_session_new(model._h, kv_block, None, 0, C.byref(h)))
+        else:
+            ids = np.ascontiguousarray(block_ids, dtype=np.uint32)
+            _check(lib.lnm_session_new(model._h, kv_block, ids.ctypes.data, ids.size, C.byref(h)))
+        self._h = h
+
+    def forward(self, tokens):
+        """Logits of the last of `tokens`, run as one batch after everything seen so far."""
+        t = np.ascontiguousarray(tokens, dtype=np.uint32)
+        logits = np.empty(self.model.hparams.n_vocab, dtype=np.float32)
+        _check(_pkg.load_library().lnm_forward(self._h, t.ctypes.data, t.size, logits.ctypes.data))
+        return logits
+
+    def generate_greedy(self, prompt, n_new):
+        """(tokens, prefill seconds, decode seconds): n_new tokens, the first from the prompt's logits."""
+        p = np.ascontiguousarray(prompt, dtype=np.uint32)
+        out = np.empty(n_new, dtype=np.uint32)
+        tp, td = C.c_double(), C.c_double()
+        _check(_pkg.load_library().lnm_generate_greedy(self._h, p.ctypes.data, p.size, n_new, out.ctypes.data,
+                                                       C.byref(tp), C.byref(td)))
+        return out, tp.value, td.value
+
+    def close(self):
+        if self._h:
+            _pkg.load_library().lnm_session_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1,0 +1,107 @@
+"""End-to-end greedy decode on the GPU against the same host code over the CPU checker.
+
+The host arithmetic (norms, RoPE, attention, SwiGLU, argmax) is shared; what differs between
+the two runs is only who computes the weight products: the HIP executor (resident matrices, or
+the content-identified dispatch layer) or the oracle's restatement of the reference's CPU
+kernels.  Identity of the generated tokens is therefore a statement about the products.
+"""
+import importlib
+
+import numpy as np
+import pytest
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def llama(pkg):
+    return importlib.import_module("llama-rust_amd.llama")
+
+
+def cpu_products(simd, threads):
+    def matmul(ty, n_rows, n_cols, n_tokens, w, x):
+        return oracle.gemm(ty, n_cols, n_tokens, w, x, n_rows, simd=simd, threads=threads)
+    return matmul
+
+
+def run_both(llama, path, prompt, n_new, simd, threads, products=None):
+    gpu = llama.Llama(path=path, products=llama.RESIDENT if products is None else products)
+    cpu = llama.Llama(path=path, products=llama.CALLBACK, matmul=cpu_products(simd, threads))
+    sg, sc = gpu.session(), cpu.session()
+    lg, lc = sg.forward(prompt), sc.forward(prompt)
+    scale = float(np.abs(lc).max())
+    worst = float(np.abs(lg - lc).max()) / scale
+    toks_g, toks_c = [llama.argmax(lg)], [llama.argmax(lc)]
+    margins = []
+    for _ in range(n_new - 1):
+        lg, lc = sg.forward([toks_g[-1]]), sc.forward([toks_c[-1]])
+        top2 = np.sort(lc)[-2:]
+        margins.append(float(top2[1] - top2[0]) / scale)
+        if toks_g[-1] == toks_c[-1]:
+            worst = max(worst, float(np.abs(lg - lc).max()) / scale)
+        toks_g.append(llama.argmax(lg))
+        toks_c.append(llama.argmax(lc))
+    return toks_g, toks_c, worst, margins
+
+
+@pytest.mark.parametrize("block_type,output_type", [(12, 14), (8, 8), (2, 6), (7, 1)])
+def test_small_model_generates_the_same_tokens_as_the_cpu_path(pkg, llama, tmp_path, block_type, output_type):
+    """Q4_K + Q6_K head (the Q4_K_M mix), Q8_0, Q4_0 + Q5_0 head, Q5_1 + F16 head."""
+    path = tmp_path / "small.gguf"
+    llama.write_synthetic_llama(path, n_layer=3, n_embd=512, n_head=8, n_head_kv=2, n_ff=1536, n_vocab=2048,
+                                block_type=block_type, embd_type=block_type, output_type=output_type, seed=11)
+    rng = np.random.default_rng(2)
+    prompt = rng.integers(0, 2048, 24).tolist()
+    toks_g, toks_c, worst, margins = run_both(llama, path, prompt, 24, simd=False, threads=1)
+    assert toks_g == toks_c, (toks_g, toks_c, min(margins))
+    assert worst <= 1e-4, worst  # logits, relative to the largest logit
+
+
+def test_dispatch_route_equals_resident_route_and_hits_its_cache(pkg, llama, tmp_path):
+    """The drop-in call shape (gemv_<t>_f32 / gemm_<t>_f32 behind the content-identified cache,
+    langtax/src/native_gpu.rs:124-213) runs the same kernels on the same bytes."""
+    path = tmp_path / "small.gguf"
+    llama.write_synthetic_llama(path, n_layer=2, n_embd=512, n_head=8, n_head_kv=4, n_ff=1024, n_vocab=1024, seed=5)
+    prompt = list(range(100, 117))
+    pkg.load_library().lnq_reset()
+    a = llama.Llama(path=path, products=llama.RESIDENT)
+    b = llama.Llama(path=path, products=llama.DISPATCH)
+    ta, _, _ = a.session().generate_greedy(prompt, 10)
+    tb, _, _ = b.session().generate_greedy(prompt, 10)
+    assert ta.tolist() == tb.tolist()
+    la, lb = a.session().forward(prompt), b.session().forward(prompt)
+    assert la.view(np.uint32).tolist() == lb.view(np.uint32).tolist()
+    st = pkg.cache_stats()
+    # 15 matrices, 11 forward passes: each matrix uploaded once, found again ten times
+    assert st["entries"] == 2 * 7 + 1 and st["misses"] == 15 and st["hits"] == 150
+
+
+def test_prompt_as_one_batch_agrees_with_token_by_token_on_the_gpu(pkg, llama, tmp_path):
+    """The batch runs the multi-token kernels, the steps the single-token ones: same values up to
+    f32 summation order."""
+    path = tmp_path / "small.gguf"
+    llama.write_synthetic_llama(path, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, n_ff=1536, n_vocab=1024, seed=9)
+    m = llama.Llama(path=path)
+    tokens = list(range(3, 3 + 37))
+    batch = m.session().forward(tokens)
+    s = m.session()
+    for t in tokens:
+        step = s.forward([t])
+    assert np.abs(batch - step).max() <= 1e-4 * np.abs(batch).max()
+    assert llama.argmax(batch) == llama.argmax(step)
+
+
+def test_8b_layer_shapes_generate_the_same_tokens_as_the_simd_cpu_path(pkg, llama, tmp_path):
+    """Two layers of the Llama-3-8B shape (d 4096, 32 / 8 heads, ffn 14336, vocab 128256, Q4_K with a
+    Q6_K head, RoPE base 5e5, K/V block 16) against the restated AVX2 kernels with the reference's
+    thread rule.  32 prompt tokens, 16 generated."""
+    path = tmp_path / "l3.gguf"
+    llama.write_synthetic_llama(path, n_layer=2, n_embd=4096, n_head=32, n_head_kv=8, n_ff=14336, n_vocab=128256,
+                                rope_base=5e5, rms_eps=1e-5, seed=1)
+    rng = np.random.default_rng(3)
+    prompt = rng.integers(0, 128256, 32).tolist()
+    toks_g, toks_c, worst, margins = run_both(llama, path, prompt, 16, simd=True, threads=0)
+    assert toks_g == toks_c, (toks_g, toks_c, min(margins))
+    assert worst <= 1e-4, worst
