@@ -206,6 +206,47 @@ def other_workloads(pkg, hip, gpu, stream, rng, cpu):
     return out
 
 
+def greedy_decode(pkg, layers, check_cpu, seed):
+    """BASELINE config 4: a random Llama-3-8B-shaped Q4_K / Q6_K-head GGUF, 128 prompt ids as one
+    batch, then 128 greedy single-token steps through the host decode (host attention and norms,
+    every weight product on the GPU with host round trips, as the reference's executor is called).
+    With check_cpu the same host code runs again over the CPU kernels and the tokens are compared."""
+    import tempfile
+    L = importlib.import_module("llama-rust_amd.llama")
+    out = {"layers": layers, "prompt_tokens": 128, "decode_steps": 128, "kv_block": 16}
+    with tempfile.TemporaryDirectory() as tmp:
+        path = os.path.join(tmp, "llama3_8b_shape.gguf")
+        t0 = time.perf_counter()
+        L.write_synthetic_llama(path, n_layer=layers, n_embd=D, n_head=32, n_head_kv=8, n_ff=FF, n_vocab=VOCAB,
+                                rope_base=5e5, rms_eps=1e-5, weight_std=0.02, seed=seed)
+        out["model_gb"] = round(os.path.getsize(path) / 1e9, 3)
+        log(f"[bench] wrote {out['model_gb']} GB GGUF in {time.perf_counter() - t0:.1f} s")
+        prompt = np.random.default_rng(seed).integers(0, VOCAB, 128)
+        m = L.Llama(path=path, products=L.RESIDENT)
+        t0 = time.perf_counter()
+        m.session().forward(prompt[:2])  # uploads every matrix
+        out["upload_s"] = round(time.perf_counter() - t0, 2)
+        sess = m.session(kv_block=16)
+        toks, prefill_s, decode_s = sess.generate_greedy(prompt, 129)
+        prod_s, att_s, n_prod = sess.timing()
+        out.update(products_s=round(prod_s, 3), attention_s=round(att_s, 3), products=n_prod)
+        out.update(prefill_s=round(prefill_s, 3), prefill_tok_per_s=round(128 / prefill_s, 1),
+                   decode_s=round(decode_s, 3), decode_tok_per_s=round(128 / decode_s, 2))
+        log(f"[bench] greedy decode: prefill {prefill_s:.2f} s, 128 steps in {decode_s:.2f} s")
+        m.close()
+        if check_cpu:
+            import oracle as O
+            c = L.Llama(path=path, products=L.CALLBACK,
+                        matmul=lambda ty, n_rows, n_cols, n_tokens, w, x:
+                        O.gemm(ty, n_cols, n_tokens, w, x, n_rows, simd=True, threads=0))
+            ctoks, cp, cd = c.session(kv_block=16).generate_greedy(prompt, 129)
+            same = int(np.sum(np.cumprod(toks == ctoks)))
+            out.update(cpu_prefill_s=round(cp, 2), cpu_decode_tok_per_s=round(128 / cd, 3), cpu_threads=O.load().lro_worker_count(D),
+                       tokens_identical=bool(same == 129), identical_prefix=same)
+            c.close()
+    return out
+
+
 TOKEN_BYTES = N_LAYERS * sum(algorithmic_bytes(Q4_K, r, c) for _, r, c, _ in LAYER) + algorithmic_bytes(Q6_K, VOCAB, D)
 
 
@@ -219,6 +260,9 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="0 skips the CPU baseline")
     ap.add_argument("--seed", type=int, default=20240531)
     ap.add_argument("--no-extras", action="store_true", help="skip the other_workloads section")
+    ap.add_argument("--e2e-layers", type=int, default=0,
+                    help="also run the end-to-end greedy decode (128 prompt + 128 steps) on a model of this many layers; 32 = config 4")
+    ap.add_argument("--e2e-check", action="store_true", help="repeat the greedy decode over the CPU kernels and compare tokens")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB copy kernel three times (known traffic for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -341,12 +385,15 @@ def main():
                                                      "frac": round(head_gbs / HBM_PEAK_GBS, 4),
                                                      "launch_us": round(head_ms * 1e3 / args.steps, 2)}},
     }
+    for m in mats:
+        m.close()
+    head.close()
     if not args.no_extras:
         log("[bench] other workloads (Q8_0 GEMV, Q4_0 prefill GEMM, MoE grouped GEMM) ...")
-        for m in mats:
-            m.close()
-        head.close()
         out["other_workloads"] = other_workloads(pkg, hip, gpu, stream, rng, args.cpu_seconds > 0)
+    if args.e2e_layers > 0:
+        log("[bench] end-to-end greedy decode ...")
+        out.setdefault("other_workloads", {})["llama_greedy_decode"] = greedy_decode(pkg, args.e2e_layers, args.e2e_check, args.seed)
     if args.cpu_seconds > 0:
         log("[bench] timing the CPU baseline ...")
         out["cpu_baseline"] = cpu_baseline(sample, x_host, args.cpu_seconds)

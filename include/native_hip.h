@@ -111,6 +111,14 @@ int lnh_gemv_once(lnh_exec *exec, const float *weights, size_t weights_len, cons
 int lnh_gemm_grouped(lnh_exec *exec, size_t n_groups, const lnh_matrix *const *mats, const size_t *tokens,
                      const float *x, size_t x_len, float *y, size_t y_len);
 
+/* Several matrices times one shared input in a single call: stands in for the back-to-back
+ * gemm calls on the same activations at langtax/src/decode.rs:2754-2790 (q, k, v) and
+ * 2968-2979 (gate, up).  x holds tokens * cols floats (all matrices have the same column
+ * count); y receives the products back to back, matrix after matrix (tokens * rows[i] each).
+ * One input copy, one launch for single-token calls, one output copy. */
+int lnh_gemm_shared(lnh_exec *exec, size_t n_mats, const lnh_matrix *const *mats, size_t tokens, const float *x,
+                    size_t x_len, float *y, size_t y_len);
+
 /* ------------------------------------------------------------------ products (device buffers) */
 
 /* The same products with x and y already in this GPU's memory, enqueued on

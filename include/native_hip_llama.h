@@ -74,6 +74,11 @@ int lnm_forward(lnm_session *session, const uint32_t *tokens, size_t n, float *l
 int lnm_generate_greedy(lnm_session *session, const uint32_t *prompt, size_t n_prompt, size_t n_new,
                         uint32_t *out, double *prefill_seconds, double *decode_seconds);
 
+/* Where a session's wall time went so far: inside weight products (host round trips included),
+ * inside RoPE + attention, and how many products it ran.  Any pointer may be NULL. */
+int lnm_session_timing(const lnm_session *session, double *products_seconds, double *attention_seconds,
+                       uint64_t *n_products);
+
 /* Building blocks, exported so that each can be checked on its own. */
 int lnm_dequant_row(uint32_t ggml_type, size_t n_cols, const uint8_t *row, size_t row_len, float *y);
 int lnm_rmsnorm(float *x, const float *w, size_t n, float eps);

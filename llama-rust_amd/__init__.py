@@ -100,6 +100,7 @@ def load_library():
         "lnh_gemm": (C.c_int, [vp, vp, sz, vp, sz, vp, sz]),
         "lnh_gemv_once": (C.c_int, [vp, vp, sz, vp, sz, vp, sz]),
         "lnh_gemm_grouped": (C.c_int, [vp, sz, pvp, psz, vp, sz, vp, sz]),
+        "lnh_gemm_shared": (C.c_int, [vp, sz, pvp, sz, vp, sz, vp, sz]),
         "lnh_gemm_device": (C.c_int, [vp, vp, sz, vp, vp, vp]),
         "lnh_gemm_grouped_device": (C.c_int, [vp, sz, pvp, psz, vp, vp, vp]),
         "lnh_gemm_batch_device": (C.c_int, [vp, sz, pvp, psz, pvp, pvp, vp]),
@@ -128,6 +129,7 @@ def load_library():
         "lnm_session_free": (None, [vp]),
         "lnm_forward": (C.c_int, [vp, vp, sz, vp]),
         "lnm_generate_greedy": (C.c_int, [vp, vp, sz, sz, vp, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+        "lnm_session_timing": (C.c_int, [vp, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_uint64)]),
         "lnm_dequant_row": (C.c_int, [u32, sz, vp, sz, vp]),
         "lnm_rmsnorm": (C.c_int, [vp, vp, sz, C.c_float]),
         "lnm_rope": (C.c_int, [vp, sz, sz, sz, C.c_float]),
@@ -292,6 +294,14 @@ class HipGemv:
         toks = (C.c_size_t * n)(*tokens)
         assert output.dtype == np.float32 and output.flags.c_contiguous
         self._check(self._lib.lnh_gemm_grouped(self._h, n, mats, toks, _ptr(x), x.size, _ptr(output), output.size))
+
+    def gemm_shared(self, matrices, tokens, input, output):
+        """Several matrices times one input of `tokens` rows; products back to back in `output`."""
+        x = _f32(input).ravel()
+        n = len(matrices)
+        mats = (C.c_void_p * n)(*[m._h for m in matrices])
+        assert output.dtype == np.float32 and output.flags.c_contiguous
+        self._check(self._lib.lnh_gemm_shared(self._h, n, mats, tokens, _ptr(x), x.size, _ptr(output), output.size))
 
     def gemm_device(self, matrix, tokens, x_ptr, y_ptr, stream=0):
         self._check(self._lib.lnh_gemm_device(self._h, matrix._h, tokens, C.c_void_p(x_ptr), C.c_void_p(y_ptr),

@@ -241,8 +241,9 @@ int check_gemm(lnh_exec *e, const lnh_matrix *m, size_t tokens, bool have_lens, 
 }
 
 // H2D x, kernel(s), blocking D2H y (native-cuda/src/gpu.rs:301-303, 332-334).
+// shared_x: every group reads the same x (tokens[0] rows of it), copied to the device once.
 int run_host(lnh_exec *e, size_t n_groups, const lnh_matrix *const *mats, const size_t *tokens, const float *x,
-             size_t x_total, float *y, size_t y_total) {
+             size_t x_total, float *y, size_t y_total, bool shared_x = false) {
     hipError_t h = hipSetDevice(e->ctx->device);
     if (h != hipSuccess) return hip_fail(e, h, "hipSetDevice");
     int rc = ensure_scratch(e, x_total, y_total);
@@ -255,7 +256,7 @@ int run_host(lnh_exec *e, size_t n_groups, const lnh_matrix *const *mats, const 
     for (size_t g = 0; g < n_groups; g++) {
         xs[g] = e->d_in + xo;
         ys[g] = e->d_out + yo;
-        xo += tokens[g] * mats[g]->view.cols;
+        if (!shared_x) xo += tokens[g] * mats[g]->view.cols;
         yo += tokens[g] * mats[g]->view.rows;
     }
     rc = launch_products(e, e->stream, n_groups, mats, tokens, xs.data(), ys.data());
@@ -436,6 +437,24 @@ static int check_groups(lnh_exec *e, size_t n_groups, const lnh_matrix *const *m
     *x_total = xt;
     *y_total = yt;
     return LNH_OK;
+}
+
+int lnh_gemm_shared(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, size_t tokens, const float *x,
+                    size_t x_len, float *y, size_t y_len) {
+    if (!e) return LNH_ERR_INVALID;
+    if (n_mats == 0 || !mats) return fail(e, LNH_ERR_INVALID, "matrix array is empty");
+    if (tokens == 0) return fail(e, LNH_ERR_INVALID, "HIP GEMM requires at least one token");
+    std::vector<size_t> toks(n_mats, tokens);
+    size_t xt, yt;
+    int rc = check_groups(e, n_mats, mats, toks.data(), &xt, &yt);
+    if (rc != LNH_OK) return rc;
+    for (size_t g = 1; g < n_mats; g++)
+        if (mats[g]->view.cols != mats[0]->view.cols)
+            return fail(e, LNH_ERR_INVALID, "matrices that share an input must have the same column count");
+    const size_t inputs = tokens * mats[0]->view.cols;
+    if (x_len != inputs || y_len != yt) return fail(e, LNH_ERR_INVALID, "HIP GEMM buffer lengths do not match shape");
+    if (!x || !y) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    return run_host(e, n_mats, mats, toks.data(), x, inputs, y, yt, true);
 }
 
 int lnh_gemm_grouped(lnh_exec *e, size_t n_groups, const lnh_matrix *const *mats, const size_t *tokens, const float *x,

@@ -11,8 +11,12 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <atomic>
 #include <chrono>
 #include <cmath>
+#include <condition_variable>
+#include <functional>
+#include <mutex>
 #include <cstdio>
 #include <cstring>
 #include <memory>
@@ -208,6 +212,72 @@ uint32_t argmax(const float *x, size_t n) {  // first maximum wins; langtax/src/
     return (uint32_t)best_i;
 }
 
+// ------------------------------------------------------------------ worker threads for the attention heads
+
+// The reference attends head after head on one thread.  Heads are independent, so they are
+// spread over a few threads here; the arithmetic of each head is untouched.
+class HeadPool {
+  public:
+    explicit HeadPool(size_t workers) {
+        for (size_t i = 0; i < workers; i++) threads_.emplace_back([this] { loop(); });
+    }
+    ~HeadPool() {
+        {
+            std::lock_guard<std::mutex> g(mu_);
+            stop_ = true;
+        }
+        wake_.notify_all();
+        for (auto &t : threads_) t.join();
+    }
+    // Calls fn(i) for every i < n, on the workers and on the calling thread; returns when all are done.
+    void run(size_t n, const std::function<void(size_t)> &fn) {
+        if (threads_.empty() || n < 2) {
+            for (size_t i = 0; i < n; i++) fn(i);
+            return;
+        }
+        {
+            std::lock_guard<std::mutex> g(mu_);
+            fn_ = &fn;
+            n_ = n;
+            next_.store(0);
+            busy_ = threads_.size();
+            epoch_++;
+        }
+        wake_.notify_all();
+        drain();
+        std::unique_lock<std::mutex> g(mu_);
+        done_.wait(g, [this] { return busy_ == 0; });
+        fn_ = nullptr;
+    }
+
+  private:
+    void drain() {
+        for (size_t i = next_.fetch_add(1); i < n_; i = next_.fetch_add(1)) (*fn_)(i);
+    }
+    void loop() {
+        uint64_t seen = 0;
+        for (;;) {
+            {
+                std::unique_lock<std::mutex> g(mu_);
+                wake_.wait(g, [&] { return stop_ || epoch_ != seen; });
+                if (stop_) return;
+                seen = epoch_;
+            }
+            drain();
+            std::lock_guard<std::mutex> g(mu_);
+            if (--busy_ == 0) done_.notify_one();
+        }
+    }
+    std::vector<std::thread> threads_;
+    std::mutex mu_;
+    std::condition_variable wake_, done_;
+    const std::function<void(size_t)> *fn_ = nullptr;
+    size_t n_ = 0, busy_ = 0;
+    std::atomic<size_t> next_{0};
+    uint64_t epoch_ = 0;
+    bool stop_ = false;
+};
+
 // ------------------------------------------------------------------ model
 
 struct Mat {
@@ -260,7 +330,12 @@ struct lnm_session {
     std::vector<uint32_t> table;      // logical block -> physical block
     std::vector<uint32_t> preset;     // physical ids to hand out, in order (empty: 0, 1, 2, ...)
     std::vector<float> cache_k, cache_v;
-    std::vector<float> x, residual, q, k, v, attn, attn_proj, gate, up, ffn_out, xn, scores;
+    // q, k, v share one buffer (matrix after matrix), and so do gate and up: products of one
+    // input can then be fetched by a single call
+    std::vector<float> x, residual, qkv, attn, attn_proj, gate_up, ffn_out, xn;
+    double products_s = 0.0, attention_s = 0.0;  // wall time spent in weight products / in attend + RoPE
+    uint64_t n_products = 0;
+    std::unique_ptr<HeadPool> pool;
 };
 
 namespace {
@@ -347,8 +422,51 @@ int finish_load(lnm_model *m) {
     return 0;
 }
 
+int product_routed(lnm_model *m, Mat &w, size_t n, const float *x, float *y);
+
+using wall_clock = std::chrono::steady_clock;
+double since(wall_clock::time_point t0) { return std::chrono::duration<double>(wall_clock::now() - t0).count(); }
+
+// One weight product of a session, timed.
+int product(lnm_session *s, Mat &w, size_t n, const float *x, float *y) {
+    const auto t0 = wall_clock::now();
+    const int rc = product_routed(s->model, w, n, x, y);
+    s->products_s += since(t0);
+    s->n_products++;
+    return rc;
+}
+
+// Several matrices times the same input; ys[i] must lie back to back in that order.
+int products_shared(lnm_session *s, std::initializer_list<Mat *> ws, size_t n, const float *x, float *y) {
+    lnm_model *m = s->model;
+    if (m->route != LNM_PRODUCTS_RESIDENT) {  // the reference's call shape: one product per call
+        for (Mat *w : ws) {
+            if (product(s, *w, n, x, y) != 0) return 1;
+            y += n * w->n_rows;
+        }
+        return 0;
+    }
+    const auto t0 = wall_clock::now();
+    if (!m->exec && lnh_create(0, &m->exec) != 0) return fail(std::string("executor: ") + lnh_thread_error());
+    const lnh_matrix *handles[4];
+    size_t k = 0, y_len = 0;
+    for (Mat *w : ws) {
+        if (!w->resident &&
+            lnh_upload_packed(m->exec, w->type, w->n_rows, w->n_cols, w->bytes, w->nbytes, &w->resident) != 0)
+            return fail(std::string(lnh_last_error(m->exec)) + " (" + w->name + ")");
+        handles[k++] = w->resident;
+        y_len += n * w->n_rows;
+    }
+    const Mat *first = *ws.begin();
+    if (lnh_gemm_shared(m->exec, k, handles, n, x, n * first->n_cols, y, y_len) != 0)
+        return fail(std::string(lnh_last_error(m->exec)) + " (" + first->name + ")");
+    s->products_s += since(t0);
+    s->n_products += k;
+    return 0;
+}
+
 // One weight product, by the model's route.
-int product(lnm_model *m, Mat &w, size_t n, const float *x, float *y) {
+int product_routed(lnm_model *m, Mat &w, size_t n, const float *x, float *y) {
     const size_t x_len = n * w.n_cols, y_len = n * w.n_rows;
     switch (m->route) {
     case LNM_PRODUCTS_CALLBACK:
@@ -408,6 +526,11 @@ int forward(lnm_session *s, const uint32_t *tokens, size_t n, float *logits) {
     const size_t d = hp.n_embd, hd = hp.head_dim, qw = (size_t)hp.n_head * hd, kvw = (size_t)hp.n_head_kv * hd;
     const size_t gqa = hp.n_head / hp.n_head_kv;
     if (ensure_blocks(s, s->past + n) != 0) return 1;
+    if (!s->pool) {
+        const unsigned hw = std::thread::hardware_concurrency();
+        const size_t threads = hw < 2 ? 1 : (hw > 16 ? 16 : hw);
+        s->pool.reset(new HeadPool(threads - 1));
+    }
     s->x.resize(n * d);
     const size_t emb_row = m->token_embd.nbytes / m->token_embd.n_rows;
     for (size_t t = 0; t < n; t++) {
@@ -415,13 +538,12 @@ int forward(lnm_session *s, const uint32_t *tokens, size_t n, float *logits) {
         if (!dequant_row(m->token_embd.type, d, m->token_embd.bytes + (size_t)tokens[t] * emb_row, &s->x[t * d]))
             return fail("cannot dequantize token_embd.weight");
     }
-    s->q.resize(n * qw);
-    s->k.resize(n * kvw);
-    s->v.resize(n * kvw);
+    s->qkv.resize(n * (qw + 2 * kvw));
+    s->gate_up.resize(2 * n * hp.n_ff);
+    float *const q = s->qkv.data(), *const k = q + n * qw, *const v = k + n * kvw;
+    float *const gate = s->gate_up.data(), *const up = gate + n * hp.n_ff;
     s->attn.resize(n * qw);
     s->attn_proj.resize(n * d);
-    s->gate.resize(n * hp.n_ff);
-    s->up.resize(n * hp.n_ff);
     s->ffn_out.resize(n * d);
     const float hd_f = hd <= 65535 ? (float)hd : 1.f;
     const float root = std::sqrt(hd_f);
@@ -431,59 +553,59 @@ int forward(lnm_session *s, const uint32_t *tokens, size_t n, float *logits) {
         Layer &l = m->layers[li];
         s->residual = s->x;
         for (size_t t = 0; t < n; t++) rmsnorm(&s->x[t * d], l.attn_norm.data(), d, hp.rms_eps);
-        if (product(m, l.wq, n, s->x.data(), s->q.data()) || product(m, l.wk, n, s->x.data(), s->k.data()) ||
-            product(m, l.wv, n, s->x.data(), s->v.data()))
-            return 1;
+        if (products_shared(s, {&l.wq, &l.wk, &l.wv}, n, s->x.data(), q)) return 1;
+        const auto t_att = wall_clock::now();
         for (size_t t = 0; t < n; t++) {  // rotate and store K, store V
             const size_t p = s->past + t;
-            float *kt = &s->k[t * kvw];
+            float *kt = k + t * kvw;
             for (size_t h = 0; h < hp.n_head_kv; h++) {
                 rope(kt + h * hd, hd, p, hp.n_rot, hp.rope_base);
                 std::memcpy(&s->cache_k[kv_offset(s, li, h, p)], kt + h * hd, hd * sizeof(float));
-                std::memcpy(&s->cache_v[kv_offset(s, li, h, p)], &s->v[t * kvw + h * hd], hd * sizeof(float));
+                std::memcpy(&s->cache_v[kv_offset(s, li, h, p)], v + t * kvw + h * hd, hd * sizeof(float));
             }
         }
-        for (size_t t = 0; t < n; t++) {  // decode.rs:11126-11197
+        // decode.rs:11126-11197, one (token, query head) pair per work item
+        const std::function<void(size_t)> attend = [&](size_t item) {
+            static thread_local std::vector<float> scores;
+            const size_t t = item / hp.n_head, hq = item % hp.n_head;
             const size_t p = s->past + t, seq = p + 1;
-            float *qt = &s->q[t * qw];
-            s->scores.resize(seq);
-            for (size_t hq = 0; hq < hp.n_head; hq++) {
-                float *qv = qt + hq * hd;
-                rope(qv, hd, p, hp.n_rot, hp.rope_base);
-                const size_t hkv = hq / gqa;
-                for (size_t u = 0; u < seq; u++) {
-                    const float *kv = &s->cache_k[kv_offset(s, li, hkv, u)];
-                    float dot = 0.f;
-                    for (size_t i = 0; i < hd; i++) dot += qv[i] * kv[i];
-                    s->scores[u] = dot * score_scale;
-                }
-                softmax(s->scores.data(), seq);
-                float *dst = &s->attn[t * qw + hq * hd];
-                for (size_t i = 0; i < hd; i++) dst[i] = 0.f;
-                for (size_t u = 0; u < seq; u++) {
-                    const float *vv = &s->cache_v[kv_offset(s, li, hkv, u)];
-                    const float st = s->scores[u];
-                    for (size_t i = 0; i < hd; i++) dst[i] += st * vv[i];
-                }
+            scores.resize(seq);
+            float *qv = q + t * qw + hq * hd;
+            rope(qv, hd, p, hp.n_rot, hp.rope_base);
+            const size_t hkv = hq / gqa;
+            for (size_t u = 0; u < seq; u++) {
+                const float *kv = &s->cache_k[kv_offset(s, li, hkv, u)];
+                float dot = 0.f;
+                for (size_t i = 0; i < hd; i++) dot += qv[i] * kv[i];
+                scores[u] = dot * score_scale;
             }
-        }
-        if (product(m, l.wo, n, s->attn.data(), s->attn_proj.data())) return 1;
+            softmax(scores.data(), seq);
+            float *dst = &s->attn[t * qw + hq * hd];
+            for (size_t i = 0; i < hd; i++) dst[i] = 0.f;
+            for (size_t u = 0; u < seq; u++) {
+                const float *vv = &s->cache_v[kv_offset(s, li, hkv, u)];
+                const float st = scores[u];
+                for (size_t i = 0; i < hd; i++) dst[i] += st * vv[i];
+            }
+        };
+        s->pool->run(n * hp.n_head, attend);
+        s->attention_s += since(t_att);
+        if (product(s, l.wo, n, s->attn.data(), s->attn_proj.data())) return 1;
         for (size_t i = 0; i < n * d; i++) s->x[i] = s->attn_proj[i] + s->residual[i];
         s->residual = s->x;
         for (size_t t = 0; t < n; t++) rmsnorm(&s->x[t * d], l.ffn_norm.data(), d, hp.rms_eps);
-        if (product(m, l.gate, n, s->x.data(), s->gate.data()) || product(m, l.up, n, s->x.data(), s->up.data()))
-            return 1;
+        if (products_shared(s, {&l.gate, &l.up}, n, s->x.data(), gate)) return 1;
         for (size_t i = 0; i < n * hp.n_ff; i++) {  // SiLU(gate) * up, decode.rs:11826-11830 and 2981-2984
-            const float g = s->gate[i];
-            s->gate[i] = g / (1.f + std::exp(-g));
-            s->gate[i] *= s->up[i];
+            const float g = gate[i];
+            gate[i] = g / (1.f + std::exp(-g));
+            gate[i] *= up[i];
         }
-        if (product(m, l.down, n, s->gate.data(), s->ffn_out.data())) return 1;
+        if (product(s, l.down, n, gate, s->ffn_out.data())) return 1;
         for (size_t i = 0; i < n * d; i++) s->x[i] = s->ffn_out[i] + s->residual[i];
     }
     s->xn.assign(s->x.begin() + (n - 1) * d, s->x.begin() + n * d);
     rmsnorm(s->xn.data(), m->output_norm.data(), d, hp.rms_eps);
-    if (product(m, m->output, 1, s->xn.data(), logits)) return 1;
+    if (product(s, m->output, 1, s->xn.data(), logits)) return 1;
     s->past += n;
     return 0;
 }
@@ -712,6 +834,15 @@ int lnm_generate_greedy(lnm_session *session, const uint32_t *prompt, size_t n_p
     const auto t2 = clock::now();
     if (prefill_seconds) *prefill_seconds = std::chrono::duration<double>(t1 - t0).count();
     if (decode_seconds) *decode_seconds = std::chrono::duration<double>(t2 - t1).count();
+    return 0;
+}
+
+int lnm_session_timing(const lnm_session *session, double *products_seconds, double *attention_seconds,
+                       uint64_t *n_products) {
+    if (!session) return fail("null argument");
+    if (products_seconds) *products_seconds = session->products_s;
+    if (attention_seconds) *attention_seconds = session->attention_s;
+    if (n_products) *n_products = session->n_products;
     return 0;
 }
 

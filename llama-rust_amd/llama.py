@@ -187,6 +187,12 @@ class Session:
                                                        C.byref(tp), C.byref(td)))
         return out, tp.value, td.value
 
+    def timing(self):
+        """(seconds in weight products, seconds in RoPE + attention, number of products) so far."""
+        a, b, n = C.c_double(), C.c_double(), C.c_uint64()
+        _check(_pkg.load_library().lnm_session_timing(self._h, C.byref(a), C.byref(b), C.byref(n)))
+        return a.value, b.value, n.value
+
     def close(self):
         if self._h:
             _pkg.load_library().lnm_session_free(self._h)

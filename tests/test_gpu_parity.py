@@ -440,6 +440,41 @@ def test_grouped_gemm_with_empty_groups_and_dispatch_layer(pkg):
         yo += t * rows
 
 
+def test_shared_input_products_equal_separate_calls(pkg, gpu):
+    """q, k, v (and gate, up) read the same activations: one call, one input copy.  The values are those
+    of the separate calls bit for bit (same kernels, same order of additions within each row)."""
+    rng = np.random.default_rng(21)
+    for ty, cols, rows_list in [(K.Q4_K, 4096, (4096, 1024, 1024)), (K.Q8_0, 1024, (256, 96)),
+                                (K.Q6_K, 512, (64, 64, 64, 64)), (K.F16, 320, (33, 7))]:
+        ws = [K.random_packed(ty, r, cols, rng) for r in rows_list]
+        mats = [gpu.upload_packed(ty, r, cols, w) for r, w in zip(rows_list, ws)]
+        for tokens in (1, 5, 40):
+            x = rng.normal(0, 1, tokens * cols).astype(np.float32)
+            y = np.full(tokens * sum(rows_list), np.nan, np.float32)
+            gpu.gemm_shared(mats, tokens, x, y)
+            off = 0
+            for r, w, m in zip(rows_list, ws, mats):
+                part = y[off:off + tokens * r]
+                check(part, ty, cols, tokens, r, w, x, f"shared {pkg.TYPE_NAMES[ty]} rows {r} tokens {tokens}")
+                alone = np.full(tokens * r, np.nan, np.float32)
+                gpu.gemm_resident(m, tokens, x, alone)
+                if tokens == 1:
+                    assert part.view(np.uint32).tolist() == alone.view(np.uint32).tolist()
+                else:  # the split of long rows over workgroups is sized by the whole launch
+                    assert np.abs(part - alone).max() <= 2e-5 * np.sqrt(np.mean(alone.astype(np.float64) ** 2))
+                off += tokens * r
+        with pytest.raises(pkg.NativeHipError, match="buffer lengths"):
+            gpu.gemm_shared(mats, 2, np.zeros(cols, np.float32), np.zeros(2 * sum(rows_list), np.float32))
+        for m in mats:
+            m.close()
+    a = gpu.upload_packed(K.Q8_0, 32, 256, K.random_packed(K.Q8_0, 32, 256, rng))
+    b = gpu.upload_packed(K.Q8_0, 32, 512, K.random_packed(K.Q8_0, 32, 512, rng))
+    with pytest.raises(pkg.NativeHipError, match="same column count"):
+        gpu.gemm_shared([a, b], 1, np.zeros(256, np.float32), np.zeros(64, np.float32))
+    with pytest.raises(pkg.NativeHipError, match="at least one token"):
+        gpu.gemm_shared([a], 0, np.zeros(0, np.float32), np.zeros(0, np.float32))
+
+
 # ------------------------------------------------------------------ residency
 def test_residency_lru_and_budget(pkg, monkeypatch):
     """langtax/src/native_gpu.rs:161-211: hit moves to the back, admission evicts from the front,
