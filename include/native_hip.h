@@ -140,6 +140,13 @@ int lnh_gemm_grouped_device(lnh_exec *exec, size_t n_groups, const lnh_matrix *c
  * layer) are issued without a host round trip each. */
 int lnh_gemm_batch_device(lnh_exec *exec, size_t n, const lnh_matrix *const *mats, const size_t *tokens,
                           const float *const *device_x, float *const *device_y, void *stream);
+/* Up to eight single-token products that read the same device_x (equal dtype and column count), one
+ * launch: device_ys[i] = mats[i] * x, or, with accumulate != 0, device_ys[i] += mats[i] * x.  The
+ * second form is the product followed by the residual addition of langtax/src/decode.rs:2957 and
+ * 3043 (x = attn_proj + residual, x = ffn_out + residual) done in the product's epilogue; a
+ * y must then not alias x.  LNH_ERR_UNSUPPORTED when a row is too long for the single-token kernels. */
+int lnh_gemv_shared_device(lnh_exec *exec, size_t n_mats, const lnh_matrix *const *mats, const float *device_x,
+                           float *const *device_ys, int accumulate, void *stream);
 /* Measurement aid, no counterpart in the reference: a plain device-to-device copy kernel
  * (nbytes a multiple of 16) whose known traffic calibrates HBM byte counters. */
 int lnh_calibration_copy(lnh_exec *exec, void *device_dst, const void *device_src, size_t nbytes, void *stream);

@@ -64,6 +64,16 @@ int lnm_set_products(lnm_model *model, int route, lnm_matmul_fn fn, void *user);
  * NULL allocates blocks in order as the sequence grows. */
 int lnm_session_new(lnm_model *model, size_t kv_block, const uint32_t *block_ids, size_t n_block_ids,
                     lnm_session **out);
+/* A session whose whole decode step stays on the GPU (needs the RESIDENT route): embedding row, RMSNorm,
+ * RoPE, attention over the paged K/V cache (device memory, same addressing), SiLU(gate)*up and the greedy
+ * pick are small kernels between the single-token products, the residual additions are done in the
+ * epilogue of the o and down products, and one step is one HIP graph whose replays pass the picked token
+ * on in device memory.  No counterpart in the reference, whose every product returns to the host
+ * (langtax/src/native_gpu.rs:124-213); the arithmetic of the small kernels is the host code's, element for
+ * element, except for the order of the sums inside RMSNorm and the softmax denominator.
+ * `max_positions` sizes the cache (rounded up to whole blocks); a batch of n tokens runs as n steps. */
+int lnm_session_new_device(lnm_model *model, size_t kv_block, const uint32_t *block_ids, size_t n_block_ids,
+                           size_t max_positions, lnm_session **out);
 void lnm_session_free(lnm_session *session);
 /* Runs the n tokens as one batch at positions past .. past+n-1 (products with n_tokens = n) and
  * writes the logits of the last one (n_vocab floats). */

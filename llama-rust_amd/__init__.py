@@ -104,6 +104,7 @@ def load_library():
         "lnh_gemm_device": (C.c_int, [vp, vp, sz, vp, vp, vp]),
         "lnh_gemm_grouped_device": (C.c_int, [vp, sz, pvp, psz, vp, vp, vp]),
         "lnh_gemm_batch_device": (C.c_int, [vp, sz, pvp, psz, pvp, pvp, vp]),
+        "lnh_gemv_shared_device": (C.c_int, [vp, sz, pvp, vp, pvp, C.c_int, vp]),
         "lnh_calibration_copy": (C.c_int, [vp, vp, vp, sz, vp]),
         "lnh_synchronize": (C.c_int, [vp]),
         "lnh_shape_checked": (C.c_int, [sz, sz, sz, sz, C.POINTER(u32), C.POINTER(u32)]),
@@ -126,6 +127,7 @@ def load_library():
         "lnm_info": (C.c_int, [vp, vp]),
         "lnm_set_products": (C.c_int, [vp, C.c_int, vp, vp]),
         "lnm_session_new": (C.c_int, [vp, sz, vp, sz, pvp]),
+        "lnm_session_new_device": (C.c_int, [vp, sz, vp, sz, sz, pvp]),
         "lnm_session_free": (None, [vp]),
         "lnm_forward": (C.c_int, [vp, vp, sz, vp]),
         "lnm_generate_greedy": (C.c_int, [vp, vp, sz, sz, vp, C.POINTER(C.c_double), C.POINTER(C.c_double)]),

@@ -537,6 +537,33 @@ int lnh_gemm_batch_device(lnh_exec *e, size_t n, const lnh_matrix *const *mats, 
     return LNH_OK;
 }
 
+int lnh_gemv_shared_device(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, const float *dx,
+                           float *const *dys, int accumulate, void *stream) {
+    if (!e) return LNH_ERR_INVALID;
+    if (n_mats == 0 || n_mats > 8) return fail(e, LNH_ERR_INVALID, "between one and eight matrices share an input");
+    if (!mats || !dx || !dys) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    nh::MatView views[8];
+    float *ys[8];
+    for (size_t i = 0; i < n_mats; i++) {
+        size_t inputs, outputs;
+        int rc = check_gemm(e, mats[i], 1, false, 0, 0, &inputs, &outputs);
+        if (rc != LNH_OK) return rc;
+        if (!dys[i]) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+        if (mats[i]->view.type != mats[0]->view.type || mats[i]->view.cols != mats[0]->view.cols)
+            return fail(e, LNH_ERR_INVALID, "matrices that share an input must share dtype and column count");
+        views[i] = mats[i]->view;
+        ys[i] = dys[i];
+    }
+    hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
+    hipError_t h = nh::launch_gemv_multi(s, views, ys, (uint32_t)n_mats, dx, accumulate != 0);
+    if (h == hipErrorInvalidValue) {
+        (void)hipGetLastError();
+        return fail(e, LNH_ERR_UNSUPPORTED, "rows too long for the single-token kernels");
+    }
+    if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
+    return LNH_OK;
+}
+
 int lnh_calibration_copy(lnh_exec *e, void *device_dst, const void *device_src, size_t nbytes, void *stream) {
     if (!e) return LNH_ERR_INVALID;
     if (!device_dst || !device_src || nbytes % 16 != 0) return fail(e, LNH_ERR_INVALID, "copy needs device pointers and a multiple of 16 bytes");

@@ -35,8 +35,9 @@ hipError_t launch_gemm_groups(hipStream_t stream, const MatView *mats, const Mat
 
 // One launch for up to 8 single-token products that read the same x and share dtype
 // and column count (q/k/v, gate/up).  hipErrorInvalidValue = not fusable this way;
-// the caller then launches them one by one.
-hipError_t launch_gemv_multi(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x);
+// the caller then launches them one by one.  accumulate: y += W x instead of y = W x.
+hipError_t launch_gemv_multi(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x,
+                             bool accumulate = false);
 
 // dst[0, nbytes) = src[0, nbytes) (nbytes a multiple of 16): reference traffic for counter calibration.
 hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t nbytes);

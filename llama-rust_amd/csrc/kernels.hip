@@ -40,7 +40,7 @@ void set_device_limits(int cu_count, size_t lds_per_block) {
 // kernel" (x too long for LDS); the caller then uses the tiled kernel.
 template <uint32_t T, int R>
 static hipError_t launch_gemv_t(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n_jobs,
-                                const float *x) {
+                                const float *x, bool accumulate) {
     constexpr int E = Geo<T>::E;
     GemvBatch b;
     const uint32_t cols = mats[0].cols;
@@ -58,7 +58,8 @@ static hipError_t launch_gemv_t(hipStream_t stream, const MatView *mats, float *
     }
     for (uint32_t j = n_jobs; j < GEMV_MAX_JOBS; j++) b.job[j] = b.job[0];
     b.total_rgs = rgs;
-    b.unit0 = b.units = b.accumulate = b.pad = 0;  // column windows are a lane-per-unit matter
+    b.unit0 = b.units = b.pad = 0;  // column windows are a lane-per-unit matter
+    b.accumulate = accumulate;
     const size_t lds = ((size_t)b.x_pad + (T == T_F32 || T == T_F16 ? 0 : 2 * (size_t)b.n_chunks)) * sizeof(float);
     if (lds > g_lds_limit) return hipErrorInvalidValue;
     auto kern = gemv_kernel<T, R>;
@@ -200,7 +201,7 @@ struct UnitWindows {
 };
 
 static hipError_t launch_gemv_q4k(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n_jobs,
-                                  const float *x) {
+                                  const float *x, bool accumulate) {
     const uint32_t nb = mats[0].nb;
     // one lane per super-block, at most 64 per row and launch: longer rows take several launches
     const UnitWindows win(nb, 64);
@@ -218,7 +219,7 @@ static hipError_t launch_gemv_q4k(hipStream_t stream, const MatView *mats, float
         const uint32_t rgs = fill_unit_jobs(b, mats, ys, n_jobs, x, lb);
         b.unit0 = win.first(w);
         b.units = units;
-        b.accumulate = w > 0;
+        b.accumulate = accumulate || w > 0;
         const size_t lds = (size_t)(64 * (lbb * 4 + 4) + lbb * 8) * sizeof(float);
         if (lds > g_lds_limit) return hipErrorInvalidValue;
         hipError_t e;
@@ -268,7 +269,7 @@ static hipError_t launch_q6k_lb(hipStream_t stream, const GemvBatch &b, uint32_t
 }
 
 static hipError_t launch_gemv_q6k(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n_jobs,
-                                  const float *x) {
+                                  const float *x, bool accumulate) {
     const uint32_t nb = mats[0].nb;
     const UnitWindows win(nb, 64);
     for (uint32_t w = 0; w < win.n; w++) {
@@ -279,7 +280,7 @@ static hipError_t launch_gemv_q6k(hipStream_t stream, const MatView *mats, float
         const uint32_t rgs = fill_unit_jobs(b, mats, ys, n_jobs, x, lb);
         b.unit0 = win.first(w);
         b.units = units;
-        b.accumulate = w > 0;
+        b.accumulate = accumulate || w > 0;
         const size_t lds = (size_t)(64 * (lb * 4 + 4)) * sizeof(float);
         if (lds > g_lds_limit) return hipErrorInvalidValue;
         hipError_t e;
@@ -325,7 +326,7 @@ static hipError_t launch_b32_lb(hipStream_t stream, const GemvBatch &b, uint32_t
 // hipErrorInvalidValue: rows are not whole units (block-order layout).
 template <uint32_t T>
 static hipError_t launch_gemv_b32(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n_jobs,
-                                  const float *x) {
+                                  const float *x, bool accumulate) {
     using G = B32Geo<T>;
     const uint32_t cols = mats[0].cols;
     if (!piece_major(T, cols)) return hipErrorInvalidValue;
@@ -343,7 +344,7 @@ static hipError_t launch_gemv_b32(hipStream_t stream, const MatView *mats, float
         const uint32_t rgs = fill_unit_jobs(b, mats, ys, n_jobs, x, lb);
         b.unit0 = win.first(w);
         b.units = units;
-        b.accumulate = w > 0;
+        b.accumulate = accumulate || w > 0;
         const size_t lds = (size_t)n_iter * ((G::UC / 4) * (lb * 4 + 4) + G::NBLK * lb) * sizeof(float);
         if (lds > g_lds_limit) return hipErrorInvalidValue;
         hipError_t e;
@@ -371,11 +372,12 @@ static hipError_t launch_tiled_t(hipStream_t stream, const MatView &m, uint32_t 
 }
 
 template <uint32_t T>
-static hipError_t launch_multi_t(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x) {
-    if constexpr (T == T_Q4_K) return launch_gemv_q4k(stream, mats, ys, n, x);
-    if constexpr (T == T_Q6_K) return launch_gemv_q6k(stream, mats, ys, n, x);
+static hipError_t launch_multi_t(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x,
+                                 bool accumulate) {
+    if constexpr (T == T_Q4_K) return launch_gemv_q4k(stream, mats, ys, n, x, accumulate);
+    if constexpr (T == T_Q6_K) return launch_gemv_q6k(stream, mats, ys, n, x, accumulate);
     if constexpr (T == T_Q8_0 || T == T_Q4_0 || T == T_Q5_0 || T == T_Q5_1) {
-        hipError_t e = launch_gemv_b32<T>(stream, mats, ys, n, x);
+        hipError_t e = launch_gemv_b32<T>(stream, mats, ys, n, x, accumulate);
         if (e != hipErrorInvalidValue) return e;
         (void)hipGetLastError();
     }
@@ -384,9 +386,9 @@ static hipError_t launch_multi_t(hipStream_t stream, const MatView *mats, float 
     size_t rows = 0;
     for (uint32_t j = 0; j < n; j++) rows += mats[j].rows;
     const size_t wavefronts = (size_t)g_cu_count * 16;
-    if (rows >= 4 * wavefronts) return launch_gemv_t<T, 4>(stream, mats, ys, n, x);
-    if (rows >= 2 * wavefronts) return launch_gemv_t<T, 2>(stream, mats, ys, n, x);
-    return launch_gemv_t<T, 1>(stream, mats, ys, n, x);
+    if (rows >= 4 * wavefronts) return launch_gemv_t<T, 4>(stream, mats, ys, n, x, accumulate);
+    if (rows >= 2 * wavefronts) return launch_gemv_t<T, 2>(stream, mats, ys, n, x, accumulate);
+    return launch_gemv_t<T, 1>(stream, mats, ys, n, x, accumulate);
 }
 
 // ---- MFMA GEMM: planning and launch
@@ -520,7 +522,7 @@ static hipError_t launch_plain(hipStream_t stream, const MatView &m, uint32_t to
     auto run = [&](auto tag) -> hipError_t {
         constexpr uint32_t T = decltype(tag)::value;
         if (tokens == 1) {
-            hipError_t e = launch_multi_t<T>(stream, &m, &y, 1, x);
+            hipError_t e = launch_multi_t<T>(stream, &m, &y, 1, x, false);
             if (e != hipErrorInvalidValue) return e;
             (void)hipGetLastError();
         }
@@ -595,20 +597,21 @@ hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t nb
     return hipGetLastError();
 }
 
-hipError_t launch_gemv_multi(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x) {
+hipError_t launch_gemv_multi(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x,
+                             bool accumulate) {
     if (n == 0) return hipSuccess;
     if (n > GEMV_MAX_JOBS) return hipErrorInvalidValue;
     for (uint32_t j = 0; j < n; j++)
         if (mats[j].type != mats[0].type || mats[j].cols != mats[0].cols || mats[j].rows == 0) return hipErrorInvalidValue;
     switch (mats[0].type) {
-    case T_F32: return launch_multi_t<T_F32>(stream, mats, ys, n, x);
-    case T_F16: return launch_multi_t<T_F16>(stream, mats, ys, n, x);
-    case T_Q4_0: return launch_multi_t<T_Q4_0>(stream, mats, ys, n, x);
-    case T_Q5_0: return launch_multi_t<T_Q5_0>(stream, mats, ys, n, x);
-    case T_Q5_1: return launch_multi_t<T_Q5_1>(stream, mats, ys, n, x);
-    case T_Q8_0: return launch_multi_t<T_Q8_0>(stream, mats, ys, n, x);
-    case T_Q4_K: return launch_multi_t<T_Q4_K>(stream, mats, ys, n, x);
-    case T_Q6_K: return launch_multi_t<T_Q6_K>(stream, mats, ys, n, x);
+    case T_F32: return launch_multi_t<T_F32>(stream, mats, ys, n, x, accumulate);
+    case T_F16: return launch_multi_t<T_F16>(stream, mats, ys, n, x, accumulate);
+    case T_Q4_0: return launch_multi_t<T_Q4_0>(stream, mats, ys, n, x, accumulate);
+    case T_Q5_0: return launch_multi_t<T_Q5_0>(stream, mats, ys, n, x, accumulate);
+    case T_Q5_1: return launch_multi_t<T_Q5_1>(stream, mats, ys, n, x, accumulate);
+    case T_Q8_0: return launch_multi_t<T_Q8_0>(stream, mats, ys, n, x, accumulate);
+    case T_Q4_K: return launch_multi_t<T_Q4_K>(stream, mats, ys, n, x, accumulate);
+    case T_Q6_K: return launch_multi_t<T_Q6_K>(stream, mats, ys, n, x, accumulate);
     default: return hipErrorInvalidValue;
     }
 }

@@ -24,6 +24,9 @@
 #include <thread>
 #include <vector>
 
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
 #include "../../include/native_hip.h"
 #include "../../include/native_hip_llama.h"
 #include "gguf.h"
@@ -324,8 +327,11 @@ struct lnm_model {
     }
 };
 
+struct DeviceDecode;  // llama_device.inc
+
 struct lnm_session {
     lnm_model *model = nullptr;
+    std::unique_ptr<DeviceDecode, void (*)(DeviceDecode *)> dev{nullptr, nullptr};  // set: the whole step runs on the GPU
     size_t kv_block = 16, past = 0;
     std::vector<uint32_t> table;      // logical block -> physical block
     std::vector<uint32_t> preset;     // physical ids to hand out, in order (empty: 0, 1, 2, ...)
@@ -734,6 +740,8 @@ void random_rows(uint32_t type, size_t n_cols, size_t n_rows, float sigma, uint6
 
 }  // namespace
 
+#include "llama_device.inc"
+
 // ------------------------------------------------------------------ C ABI
 
 extern "C" {
@@ -810,10 +818,24 @@ int lnm_session_new(lnm_model *model, size_t kv_block, const uint32_t *block_ids
     return 0;
 }
 
+int lnm_session_new_device(lnm_model *model, size_t kv_block, const uint32_t *block_ids, size_t n_block_ids,
+                           size_t max_positions, lnm_session **out) {
+    lnm_session *s = nullptr;
+    if (lnm_session_new(model, kv_block, block_ids, n_block_ids, &s) != 0) return 1;
+    if (device_decode_create(s, max_positions) != 0) {
+        delete s;
+        *out = nullptr;
+        return 1;
+    }
+    *out = s;
+    return 0;
+}
+
 void lnm_session_free(lnm_session *session) { delete session; }
 
 int lnm_forward(lnm_session *session, const uint32_t *tokens, size_t n, float *logits) {
     if (!session || !tokens || !logits) return fail("null argument");
+    if (session->dev) return device_forward(session, tokens, n, logits);
     return forward(session, tokens, n, logits);
 }
 
@@ -821,6 +843,7 @@ int lnm_generate_greedy(lnm_session *session, const uint32_t *prompt, size_t n_p
                         uint32_t *out, double *prefill_seconds, double *decode_seconds) {
     if (!session || !prompt || !out) return fail("null argument");
     if (n_prompt == 0 || n_new == 0) return fail("empty prompt or nothing to generate");
+    if (session->dev) return device_generate(session, prompt, n_prompt, n_new, out, prefill_seconds, decode_seconds);
     std::vector<float> logits(session->model->hp.n_vocab);
     using clock = std::chrono::steady_clock;
     const auto t0 = clock::now();

@@ -144,8 +144,9 @@ class Llama:
         _check(lib.lnm_set_products(self._h, route, C.cast(cb, C.c_void_p) if cb else None, None))
         self._cb = cb  # keep the thunk alive
 
-    def session(self, kv_block=16, block_ids=None):
-        return Session(self, kv_block, block_ids)
+    def session(self, kv_block=16, block_ids=None, device_positions=None):
+        """device_positions: keep the whole decode step on the GPU, with a cache of that many positions."""
+        return Session(self, kv_block, block_ids, device_positions)
 
     def close(self):
         if self._h:
@@ -160,15 +161,16 @@ class Llama:
 
 
 class Session:
-    def __init__(self, model, kv_block=16, block_ids=None):
+    def __init__(self, model, kv_block=16, block_ids=None, device_positions=None):
         lib = _pkg.load_library()
         self.model = model
         h = C.c_void_p()
-        if block_ids is None:
-            _check(lib.lnm_session_new(model._h, kv_block, None, 0, C.byref(h)))
+        ids = None if block_ids is None else np.ascontiguousarray(block_ids, dtype=np.uint32)
+        ids_p, ids_n = (None, 0) if ids is None else (ids.ctypes.data, ids.size)
+        if device_positions is None:
+            _check(lib.lnm_session_new(model._h, kv_block, ids_p, ids_n, C.byref(h)))
         else:
-            ids = np.ascontiguousarray(block_ids, dtype=np.uint32)
-            _check(lib.lnm_session_new(model._h, kv_block, ids.ctypes.data, ids.size, C.byref(h)))
+            _check(lib.lnm_session_new_device(model._h, kv_block, ids_p, ids_n, device_positions, C.byref(h)))
         self._h = h
 
     def forward(self, tokens):
