@@ -233,6 +233,16 @@ def greedy_decode(pkg, layers, check_cpu, seed):
         out.update(prefill_s=round(prefill_s, 3), prefill_tok_per_s=round(128 / prefill_s, 1),
                    decode_s=round(decode_s, 3), decode_tok_per_s=round(128 / decode_s, 2))
         log(f"[bench] greedy decode: prefill {prefill_s:.2f} s, 128 steps in {decode_s:.2f} s")
+        # The same model with the whole step resident on the GPU (one HIP graph per token, no host round trips).
+        dev = m.session(kv_block=16, device_positions=256)
+        dtoks, dp, dd = dev.generate_greedy(prompt, 129)
+        dsame = int(np.sum(np.cumprod(toks == dtoks)))
+        out["device_session"] = {"prefill_s": round(dp, 3), "prefill_tok_per_s": round(128 / dp, 1),
+                                 "decode_s": round(dd, 4), "decode_tok_per_s": round(128 / dd, 1),
+                                 "ms_per_token": round(dd / 128 * 1e3, 3),
+                                 "tokens_identical_to_host_session": bool(dsame == 129), "identical_prefix": dsame}
+        log(f"[bench] device session: prompt token by token {dp:.2f} s, 128 steps in {dd:.3f} s ({128 / dd:.0f} tok/s)")
+        dev.close()
         m.close()
         if check_cpu:
             import oracle as O
@@ -243,6 +253,8 @@ def greedy_decode(pkg, layers, check_cpu, seed):
             same = int(np.sum(np.cumprod(toks == ctoks)))
             out.update(cpu_prefill_s=round(cp, 2), cpu_decode_tok_per_s=round(128 / cd, 3), cpu_threads=O.load().lro_worker_count(D),
                        tokens_identical=bool(same == 129), identical_prefix=same)
+            dsame_cpu = int(np.sum(np.cumprod(dtoks == ctoks)))
+            out["device_session"].update(tokens_identical_to_cpu_path=bool(dsame_cpu == 129), identical_prefix_cpu=dsame_cpu)
             c.close()
     return out
 
