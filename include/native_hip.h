@@ -147,6 +147,17 @@ int lnh_gemm_batch_device(lnh_exec *exec, size_t n, const lnh_matrix *const *mat
  * y must then not alias x.  LNH_ERR_UNSUPPORTED when a row is too long for the single-token kernels. */
 int lnh_gemv_shared_device(lnh_exec *exec, size_t n_mats, const lnh_matrix *const *mats, const float *device_x,
                            float *const *device_ys, int accumulate, void *stream);
+/* The same launch with the operation that precedes the product in the decode graph applied to x as the
+ * kernel stages it (x itself is left as it is):
+ *   LNH_PROLOGUE_RMSNORM  x := x * inv_rms(x, eps) * x2, x2 = norm weights   (langtax/src/decode.rs:11498-11513,
+ *                         called at 2745 and 2960 before the q/k/v and gate/up products)
+ *   LNH_PROLOGUE_SWIGLU   x := SiLU(x) * x2, x = gate, x2 = up               (decode.rs:11826-11830, 2981-2984)
+ * LNH_ERR_UNSUPPORTED (nothing launched) unless the matrices are Q4_K with rows of at most 16384 columns:
+ * the caller then runs the operation as a kernel of its own and calls lnh_gemv_shared_device. */
+enum { LNH_PROLOGUE_NONE = 0, LNH_PROLOGUE_RMSNORM = 1, LNH_PROLOGUE_SWIGLU = 2 };
+int lnh_gemv_fused_device(lnh_exec *exec, size_t n_mats, const lnh_matrix *const *mats, const float *device_x,
+                          float *const *device_ys, int accumulate, int prologue, const float *device_x2, float eps,
+                          void *stream);
 /* Measurement aid, no counterpart in the reference: a plain device-to-device copy kernel
  * (nbytes a multiple of 16) whose known traffic calibrates HBM byte counters. */
 int lnh_calibration_copy(lnh_exec *exec, void *device_dst, const void *device_src, size_t nbytes, void *stream);

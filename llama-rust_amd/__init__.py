@@ -36,6 +36,7 @@ TYPE_NAMES = {F32: "f32", F16: "f16", Q4_0: "q4_0", Q5_0: "q5_0", Q5_1: "q5_1", 
               Q4_K: "q4_k", Q6_K: "q6_k"}
 
 OK, ERR_INVALID, ERR_DEVICE, ERR_OOM, ERR_FOREIGN, ERR_UNSUPPORTED = range(6)
+PROLOGUE_NONE, PROLOGUE_RMSNORM, PROLOGUE_SWIGLU = 0, 1, 2
 
 
 class NativeHipError(RuntimeError):
@@ -105,6 +106,7 @@ def load_library():
         "lnh_gemm_grouped_device": (C.c_int, [vp, sz, pvp, psz, vp, vp, vp]),
         "lnh_gemm_batch_device": (C.c_int, [vp, sz, pvp, psz, pvp, pvp, vp]),
         "lnh_gemv_shared_device": (C.c_int, [vp, sz, pvp, vp, pvp, C.c_int, vp]),
+        "lnh_gemv_fused_device": (C.c_int, [vp, sz, pvp, vp, pvp, C.c_int, C.c_int, vp, C.c_float, vp]),
         "lnh_calibration_copy": (C.c_int, [vp, vp, vp, sz, vp]),
         "lnh_synchronize": (C.c_int, [vp]),
         "lnh_shape_checked": (C.c_int, [sz, sz, sz, sz, C.POINTER(u32), C.POINTER(u32)]),
@@ -325,6 +327,22 @@ class HipGemv:
     def gemm_batch_device(self, batch, stream=0):
         n, mats, toks, xs, ys = batch
         self._check(self._lib.lnh_gemm_batch_device(self._h, n, mats, toks, xs, ys, C.c_void_p(stream)))
+
+    def gemv_shared_device(self, matrices, x_ptr, y_ptrs, accumulate=False, stream=0):
+        """y_i = W_i x (accumulate: y_i += W_i x) for matrices that read the same device x, one launch."""
+        n = len(matrices)
+        mats = (C.c_void_p * n)(*[m._h for m in matrices])
+        ys = (C.c_void_p * n)(*y_ptrs)
+        self._check(self._lib.lnh_gemv_shared_device(self._h, n, mats, C.c_void_p(x_ptr), ys, int(accumulate),
+                                                     C.c_void_p(stream)))
+
+    def gemv_fused_device(self, matrices, x_ptr, y_ptrs, prologue, x2_ptr, eps=0.0, accumulate=False, stream=0):
+        """The same with PROLOGUE_RMSNORM / PROLOGUE_SWIGLU applied to x as the kernel stages it."""
+        n = len(matrices)
+        mats = (C.c_void_p * n)(*[m._h for m in matrices])
+        ys = (C.c_void_p * n)(*y_ptrs)
+        self._check(self._lib.lnh_gemv_fused_device(self._h, n, mats, C.c_void_p(x_ptr), ys, int(accumulate), prologue,
+                                                    C.c_void_p(x2_ptr), eps, C.c_void_p(stream)))
 
     def calibration_copy(self, dst_ptr, src_ptr, nbytes, stream=0):
         self._check(self._lib.lnh_calibration_copy(self._h, C.c_void_p(dst_ptr), C.c_void_p(src_ptr), nbytes,

@@ -537,11 +537,15 @@ int lnh_gemm_batch_device(lnh_exec *e, size_t n, const lnh_matrix *const *mats, 
     return LNH_OK;
 }
 
-int lnh_gemv_shared_device(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, const float *dx,
-                           float *const *dys, int accumulate, void *stream) {
+// Shared checks and launch of the single-token device products.
+static int gemv_shared_device(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, const float *dx, float *const *dys,
+                              int accumulate, int prologue, const float *dx2, float eps, void *stream) {
     if (!e) return LNH_ERR_INVALID;
     if (n_mats == 0 || n_mats > 8) return fail(e, LNH_ERR_INVALID, "between one and eight matrices share an input");
     if (!mats || !dx || !dys) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    if (prologue != LNH_PROLOGUE_NONE && prologue != LNH_PROLOGUE_RMSNORM && prologue != LNH_PROLOGUE_SWIGLU)
+        return fail(e, LNH_ERR_INVALID, "unknown prologue");
+    if (prologue != LNH_PROLOGUE_NONE && !dx2) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
     nh::MatView views[8];
     float *ys[8];
     for (size_t i = 0; i < n_mats; i++) {
@@ -555,13 +559,26 @@ int lnh_gemv_shared_device(lnh_exec *e, size_t n_mats, const lnh_matrix *const *
         ys[i] = dys[i];
     }
     hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
-    hipError_t h = nh::launch_gemv_multi(s, views, ys, (uint32_t)n_mats, dx, accumulate != 0);
+    const hipError_t h = prologue == LNH_PROLOGUE_NONE
+                             ? nh::launch_gemv_multi(s, views, ys, (uint32_t)n_mats, dx, accumulate != 0)
+                             : nh::launch_gemv_multi_prologue(s, views, ys, (uint32_t)n_mats, dx, accumulate != 0, prologue, dx2, eps);
     if (h == hipErrorInvalidValue) {
         (void)hipGetLastError();
-        return fail(e, LNH_ERR_UNSUPPORTED, "rows too long for the single-token kernels");
+        return fail(e, LNH_ERR_UNSUPPORTED, prologue == LNH_PROLOGUE_NONE ? "rows too long for the single-token kernels"
+                                                                         : "no fused prologue for this dtype or row length");
     }
     if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
     return LNH_OK;
+}
+
+int lnh_gemv_shared_device(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, const float *dx,
+                           float *const *dys, int accumulate, void *stream) {
+    return gemv_shared_device(e, n_mats, mats, dx, dys, accumulate, LNH_PROLOGUE_NONE, nullptr, 0.f, stream);
+}
+
+int lnh_gemv_fused_device(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, const float *dx, float *const *dys,
+                          int accumulate, int prologue, const float *dx2, float eps, void *stream) {
+    return gemv_shared_device(e, n_mats, mats, dx, dys, accumulate, prologue, dx2, eps, stream);
 }
 
 int lnh_calibration_copy(lnh_exec *e, void *device_dst, const void *device_src, size_t nbytes, void *stream) {

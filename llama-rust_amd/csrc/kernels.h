@@ -39,6 +39,13 @@ hipError_t launch_gemm_groups(hipStream_t stream, const MatView *mats, const Mat
 hipError_t launch_gemv_multi(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x,
                              bool accumulate = false);
 
+// The same launch with a prologue applied to x on its way into LDS (Q4_K matrices whose rows fit one
+// launch; hipErrorInvalidValue otherwise, nothing launched):
+//   prologue 1: x := x * inv_rms(x, eps) * x2   (RMSNorm, x2 = norm weights)
+//   prologue 2: x := SiLU(x) * x2               (x = gate, x2 = up)
+hipError_t launch_gemv_multi_prologue(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x,
+                                      bool accumulate, int prologue, const float *x2, float eps);
+
 // dst[0, nbytes) = src[0, nbytes) (nbytes a multiple of 16): reference traffic for counter calibration.
 hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t nbytes);
 

@@ -60,6 +60,8 @@ static hipError_t launch_gemv_t(hipStream_t stream, const MatView *mats, float *
     b.total_rgs = rgs;
     b.unit0 = b.units = b.pad = 0;  // column windows are a lane-per-unit matter
     b.accumulate = accumulate;
+    b.x2 = nullptr;
+    b.eps = 0.f;
     const size_t lds = ((size_t)b.x_pad + (T == T_F32 || T == T_F16 ? 0 : 2 * (size_t)b.n_chunks)) * sizeof(float);
     if (lds > g_lds_limit) return hipErrorInvalidValue;
     auto kern = gemv_kernel<T, R>;
@@ -144,9 +146,10 @@ hipError_t probe_fp8_nibble_unit(hipStream_t stream, float *unit_out) {
 static float g_nib_mul = 0.f;  // 1 / (value of fp8 byte 0x01); 0 = fp8 unpack not usable
 void set_fp8_nibble_unit(float unit) { g_nib_mul = unit > 0.f ? 1.0f / unit : 0.f; }
 
-template <int LB, int NW, int PL>
+template <int LB, int NW, int PL, int PRO>
 static hipError_t launch_q4k_lb(hipStream_t stream, const GemvBatch &b, uint32_t units, size_t lds) {
     const bool fp8 = g_nib_mul != 0.f;
+    if (PRO != PRO_NONE && !fp8) return hipErrorInvalidValue;  // prologues are built for the fp8 unpack only
     size_t per_cu = g_lds_limit * 2 / (lds ? lds : 1);  // 160 KB of LDS per CU
     if (per_cu < 1) per_cu = 1;
     if (per_cu > 32 / NW) per_cu = 32 / NW;             // 32 wavefronts per CU (measured +2.5 % on the decode step over 16)
@@ -154,9 +157,12 @@ static hipError_t launch_q4k_lb(hipStream_t stream, const GemvBatch &b, uint32_t
     const uint32_t needed = (units + NW - 1) / NW;
     if (grid > needed) grid = needed;
     const bool one = grid == needed;  // a wavefront for every unit
-    void (*kern)(GemvBatch, float) =
-        fp8 ? (one ? gemv_q4k_kernel<LB, NW, true, PL, true> : gemv_q4k_kernel<LB, NW, true, PL, false>)
-            : (one ? gemv_q4k_kernel<LB, NW, false, PL, true> : gemv_q4k_kernel<LB, NW, false, PL, false>);
+    void (*kern)(GemvBatch, float);
+    if constexpr (PRO == PRO_NONE)
+        kern = fp8 ? (one ? gemv_q4k_kernel<LB, NW, true, PL, true> : gemv_q4k_kernel<LB, NW, true, PL, false>)
+                   : (one ? gemv_q4k_kernel<LB, NW, false, PL, true> : gemv_q4k_kernel<LB, NW, false, PL, false>);
+    else
+        kern = one ? gemv_q4k_kernel<LB, NW, true, PL, true, PRO> : gemv_q4k_kernel<LB, NW, true, PL, false, PRO>;
     static size_t configured[4] = {0, 0, 0, 0};
     size_t &conf = configured[2 * fp8 + one];
     if (lds > 48 * 1024 && lds > conf) {
@@ -174,6 +180,9 @@ static uint32_t fill_unit_jobs(GemvBatch &b, const MatView *mats, float *const *
                                uint32_t lb) {
     const uint32_t rg_rows = 64 / lb;
     b.x = x;
+    b.x2 = nullptr;
+    b.eps = 0.f;
+    b.pad2 = 0;
     b.n_jobs = n_jobs;
     b.n_chunks = 0;
     b.x_pad = mats[0].cols;
@@ -200,11 +209,19 @@ struct UnitWindows {
     uint32_t count(uint32_t w, uint32_t nu) const { return first(w) + per <= nu ? per : nu - first(w); }
 };
 
-static hipError_t launch_gemv_q4k(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n_jobs,
-                                  const float *x, bool accumulate) {
+struct GemvPrologue {
+    int kind = PRO_NONE;        // PRO_RMSNORM: x2 = norm weights; PRO_SWIGLU: x2 = the up vector (x is gate)
+    const float *x2 = nullptr;
+    float eps = 0.f;
+};
+
+template <int PRO>
+static hipError_t launch_gemv_q4k_pro(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n_jobs,
+                                      const float *x, bool accumulate, const GemvPrologue &pro) {
     const uint32_t nb = mats[0].nb;
     // one lane per super-block, at most 64 per row and launch: longer rows take several launches
     const UnitWindows win(nb, 64);
+    if (PRO != PRO_NONE && win.n != 1) return hipErrorInvalidValue;  // a prologue needs all of x in one workgroup
     for (uint32_t w = 0; w < win.n; w++) {
         const uint32_t units = win.count(w, nb);
         uint32_t lbb = 1;  // super-blocks per row, rounded up to a power of two
@@ -220,32 +237,45 @@ static hipError_t launch_gemv_q4k(hipStream_t stream, const MatView *mats, float
         b.unit0 = win.first(w);
         b.units = units;
         b.accumulate = accumulate || w > 0;
-        const size_t lds = (size_t)(64 * (lbb * 4 + 4) + lbb * 8) * sizeof(float);
+        b.x2 = pro.x2;
+        b.eps = pro.eps;
+        // x slots, the sub-block sums of x, and room for one partial sum per wavefront (RMSNorm prologue)
+        const size_t lds = (size_t)(64 * (lbb * 4 + 4) + lbb * 8 + 16) * sizeof(float);
         if (lds > g_lds_limit) return hipErrorInvalidValue;
         hipError_t e;
         if (halves) {
             switch (lb) {
-            case 2: e = launch_q4k_lb<2, 4, 4>(stream, b, rgs, lds); break;
-            case 4: e = launch_q4k_lb<4, 4, 4>(stream, b, rgs, lds); break;
-            case 8: e = launch_q4k_lb<8, 4, 4>(stream, b, rgs, lds); break;
-            case 16: e = launch_q4k_lb<16, 4, 4>(stream, b, rgs, lds); break;
-            default: e = launch_q4k_lb<32, 4, 4>(stream, b, rgs, lds); break;
+            case 2: e = launch_q4k_lb<2, 4, 4, PRO>(stream, b, rgs, lds); break;
+            case 4: e = launch_q4k_lb<4, 4, 4, PRO>(stream, b, rgs, lds); break;
+            case 8: e = launch_q4k_lb<8, 4, 4, PRO>(stream, b, rgs, lds); break;
+            case 16: e = launch_q4k_lb<16, 4, 4, PRO>(stream, b, rgs, lds); break;
+            default: e = launch_q4k_lb<32, 4, 4, PRO>(stream, b, rgs, lds); break;
             }
         } else {
             switch (lb) {
             // Short rows: small workgroups, so that even a 1024-row matrix spreads over every CU.
-            case 1: e = launch_q4k_lb<1, 4, 8>(stream, b, rgs, lds); break;
-            case 2: e = launch_q4k_lb<2, 4, 8>(stream, b, rgs, lds); break;
-            case 4: e = launch_q4k_lb<4, 4, 8>(stream, b, rgs, lds); break;
-            case 8: e = launch_q4k_lb<8, 4, 8>(stream, b, rgs, lds); break;
-            case 16: e = launch_q4k_lb<16, 4, 8>(stream, b, rgs, lds); break;
-            case 32: e = launch_q4k_lb<32, 8, 8>(stream, b, rgs, lds); break;
-            default: e = launch_q4k_lb<64, 8, 8>(stream, b, rgs, lds); break;
+            case 1: e = launch_q4k_lb<1, 4, 8, PRO>(stream, b, rgs, lds); break;
+            case 2: e = launch_q4k_lb<2, 4, 8, PRO>(stream, b, rgs, lds); break;
+            case 4: e = launch_q4k_lb<4, 4, 8, PRO>(stream, b, rgs, lds); break;
+            case 8: e = launch_q4k_lb<8, 4, 8, PRO>(stream, b, rgs, lds); break;
+            case 16: e = launch_q4k_lb<16, 4, 8, PRO>(stream, b, rgs, lds); break;
+            case 32: e = launch_q4k_lb<32, 8, 8, PRO>(stream, b, rgs, lds); break;
+            default: e = launch_q4k_lb<64, 8, 8, PRO>(stream, b, rgs, lds); break;
             }
         }
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
+}
+
+static hipError_t launch_gemv_q4k(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n_jobs,
+                                  const float *x, bool accumulate, const GemvPrologue &pro = GemvPrologue()) {
+    switch (pro.kind) {
+    case PRO_NONE: return launch_gemv_q4k_pro<PRO_NONE>(stream, mats, ys, n_jobs, x, accumulate, pro);
+    case PRO_RMSNORM: return launch_gemv_q4k_pro<PRO_RMSNORM>(stream, mats, ys, n_jobs, x, accumulate, pro);
+    case PRO_SWIGLU: return launch_gemv_q4k_pro<PRO_SWIGLU>(stream, mats, ys, n_jobs, x, accumulate, pro);
+    default: return hipErrorInvalidValue;
+    }
 }
 
 template <int LB, int NW>
@@ -614,6 +644,19 @@ hipError_t launch_gemv_multi(hipStream_t stream, const MatView *mats, float *con
     case T_Q6_K: return launch_multi_t<T_Q6_K>(stream, mats, ys, n, x, accumulate);
     default: return hipErrorInvalidValue;
     }
+}
+
+hipError_t launch_gemv_multi_prologue(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x,
+                                      bool accumulate, int prologue, const float *x2, float eps) {
+    if (n == 0 || n > GEMV_MAX_JOBS || !x2) return hipErrorInvalidValue;
+    if (prologue != PRO_RMSNORM && prologue != PRO_SWIGLU) return hipErrorInvalidValue;
+    for (uint32_t j = 0; j < n; j++)
+        if (mats[j].type != T_Q4_K || mats[j].cols != mats[0].cols || mats[j].rows == 0) return hipErrorInvalidValue;
+    GemvPrologue pro;
+    pro.kind = prologue;
+    pro.x2 = x2;
+    pro.eps = eps;
+    return launch_gemv_q4k(stream, mats, ys, n, x, accumulate, pro);
 }
 
 hipError_t launch_gemm(hipStream_t stream, const MatView &m, const MatView &tiled, uint32_t tokens, const float *x,

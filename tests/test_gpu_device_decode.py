@@ -86,3 +86,104 @@ def test_device_session_8b_layer_shapes_against_the_simd_cpu_path(pkg, llama, tm
     gpu = llama.Llama(path=path)
     td, _, _ = gpu.session(device_positions=64).generate_greedy(prompt, 12)
     assert td.tolist() == tc.tolist()
+
+
+# ------------------------------------------------------------------ the fused prologues on their own
+
+def _device(hip, a):
+    return hip.DeviceBuffer.from_numpy(np.ascontiguousarray(a, dtype=np.float32))
+
+
+@pytest.mark.parametrize("rows,cols", [((4096, 1024, 1024), 4096), ((14336, 14336), 4096), ((4096,), 14336), ((300,), 512)])
+def test_rmsnorm_prologue_equals_rmsnorm_then_product(pkg, rows, cols):
+    """W (x * inv_rms(x) * g) with the norm done while the kernel stages x, against the float64 value of
+    the same expression on the dequantized weights, inside the f32 summation bound of the product."""
+    import cases as K
+    hip = importlib.import_module("llama-rust_amd.hiprt")
+    rng = np.random.default_rng(cols + len(rows))
+    gpu = pkg.HipGemv(0)
+    ws = [K.random_packed(K.Q4_K, r, cols, rng, signed=False, scale=0.02) for r in rows]
+    mats = [gpu.upload_packed(K.Q4_K, r, cols, w) for r, w in zip(rows, ws)]
+    x = rng.normal(0, 3.0, cols).astype(np.float32)
+    g = (1 + rng.normal(0, 0.05, cols)).astype(np.float32)
+    eps = 1e-5
+    dx, dg = _device(hip, x), _device(hip, g)
+    ys = [hip.DeviceBuffer(4 * r) for r in rows]
+    for y in ys:
+        y.fill_byte(0xff)
+    gpu.gemv_fused_device(mats, dx.ptr, [y.ptr for y in ys], pkg.PROLOGUE_RMSNORM, dg.ptr, eps)
+    gpu.synchronize()
+    x64 = x.astype(np.float64)
+    xn = x64 / np.sqrt(np.mean(x64 * x64) + eps) * g.astype(np.float64)
+    for r, w, y in zip(rows, ws, ys):
+        exact, mag = oracle.gemm_f64_mag(K.Q4_K, cols, 1, w, xn.astype(np.float32), r)
+        # the f32 roundings of the normalised x (tree sum of squares, sqrt, two multiplies) on top of the product's bound
+        exact64 = oracle.dequant(K.Q4_K, cols, w, r).astype(np.float64) @ xn
+        got = y.to_numpy(np.float32)
+        bound = K.single_kernel_bound(cols, mag.ravel()) + 16 * 2.0 ** -24 * mag.ravel()
+        assert np.all(np.abs(got - exact64) <= bound), float(np.max(np.abs(got - exact64) / bound))
+    # x itself is untouched
+    assert dx.to_numpy(np.float32).view(np.uint32).tolist() == x.view(np.uint32).tolist()
+    gpu.close()
+
+
+def test_swiglu_prologue_accumulates_like_the_separate_steps(pkg):
+    """x_res += W (SiLU(gate) * up), against float64 on the dequantized weights."""
+    import cases as K
+    hip = importlib.import_module("llama-rust_amd.hiprt")
+    rng = np.random.default_rng(77)
+    rows, cols = 4096, 14336
+    gpu = pkg.HipGemv(0)
+    w = K.random_packed(K.Q4_K, rows, cols, rng, signed=False, scale=0.02)
+    m = gpu.upload_packed(K.Q4_K, rows, cols, w)
+    gate = rng.normal(0, 2.0, cols).astype(np.float32)
+    up = rng.normal(0, 1.0, cols).astype(np.float32)
+    res = rng.normal(0, 1.0, rows).astype(np.float32)
+    dgate, dup, dres = _device(hip, gate), _device(hip, up), _device(hip, res)
+    gpu.gemv_fused_device([m], dgate.ptr, [dres.ptr], pkg.PROLOGUE_SWIGLU, dup.ptr, accumulate=True)
+    gpu.synchronize()
+    g64 = gate.astype(np.float64)
+    h = g64 / (1 + np.exp(-g64)) * up.astype(np.float64)
+    exact, mag = oracle.gemm_f64_mag(K.Q4_K, cols, 1, w, h.astype(np.float32), rows)
+    exact64 = oracle.dequant(K.Q4_K, cols, w, rows).astype(np.float64) @ h + res.astype(np.float64)
+    got = dres.to_numpy(np.float32)
+    bound = K.single_kernel_bound(cols, mag.ravel()) + 8 * 2.0 ** -24 * (mag.ravel() + np.abs(exact64))
+    assert np.all(np.abs(got - exact64) <= bound), float(np.max(np.abs(got - exact64) / bound))
+    gpu.close()
+
+
+def test_prologue_is_refused_where_it_is_not_built(pkg):
+    """Other dtypes and rows longer than one launch: LNH_ERR_UNSUPPORTED, nothing written."""
+    import cases as K
+    hip = importlib.import_module("llama-rust_amd.hiprt")
+    rng = np.random.default_rng(5)
+    gpu = pkg.HipGemv(0)
+    for ty, rows, cols in ((K.Q8_0, 64, 4096), (K.Q6_K, 64, 4096), (K.Q4_K, 16, 32768)):
+        m = gpu.upload_packed(ty, rows, cols, K.random_packed(ty, rows, cols, rng, signed=False, scale=0.02))
+        dx, dg = _device(hip, np.ones(cols)), _device(hip, np.ones(cols))
+        y = hip.DeviceBuffer(4 * rows)
+        y.fill_byte(0x5a)
+        with pytest.raises(pkg.NativeHipError) as ei:
+            gpu.gemv_fused_device([m], dx.ptr, [y.ptr], pkg.PROLOGUE_RMSNORM, dg.ptr, 1e-5)
+        assert ei.value.code == pkg.ERR_UNSUPPORTED
+        gpu.synchronize()
+        assert set(y.to_numpy(np.uint8).tolist()) == {0x5a}
+    gpu.close()
+
+
+def test_fused_and_unfused_device_sessions_agree(pkg, llama, tmp_path, monkeypatch):
+    """LLAMA_HIP_DECODE_UNFUSED keeps RMSNorm and SiLU*up as kernels of their own: same tokens, logits to 1e-4."""
+    path = tmp_path / "small.gguf"
+    llama.write_synthetic_llama(path, n_layer=3, n_embd=512, n_head=8, n_head_kv=2, n_ff=1536, n_vocab=2048, seed=33)
+    m = llama.Llama(path=path)
+    prompt = list(range(7, 7 + 15))
+    fused = m.session(device_positions=48)
+    monkeypatch.setenv("LLAMA_HIP_DECODE_UNFUSED", "1")
+    plain = m.session(device_positions=48)
+    monkeypatch.delenv("LLAMA_HIP_DECODE_UNFUSED")
+    la, lb = fused.forward(prompt), plain.forward(prompt)
+    assert logits_close(la, lb)
+    ta, _, _ = m.session(device_positions=48).generate_greedy(prompt, 16)
+    monkeypatch.setenv("LLAMA_HIP_DECODE_UNFUSED", "1")
+    tb, _, _ = m.session(device_positions=48).generate_greedy(prompt, 16)
+    assert ta.tolist() == tb.tolist()
