@@ -272,9 +272,11 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="0 skips the CPU baseline")
     ap.add_argument("--seed", type=int, default=20240531)
     ap.add_argument("--no-extras", action="store_true", help="skip the other_workloads section")
-    ap.add_argument("--e2e-layers", type=int, default=0,
-                    help="also run the end-to-end greedy decode (128 prompt + 128 steps) on a model of this many layers; 32 = config 4")
-    ap.add_argument("--e2e-check", action="store_true", help="repeat the greedy decode over the CPU kernels and compare tokens")
+    ap.add_argument("--e2e-layers", type=int, default=32,
+                    help="layers of the model of the end-to-end greedy decode (128 prompt + 128 steps); 32 = BASELINE config 4, 0 skips it")
+    ap.add_argument("--e2e-check", action="store_true", default=True,
+                    help="repeat the greedy decode over the CPU kernels and compare tokens (default)")
+    ap.add_argument("--no-e2e-check", dest="e2e_check", action="store_false")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB copy kernel three times (known traffic for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -387,6 +389,7 @@ def main():
                    "launch_mode": "eager" if args.no_graph else "hip_graph"},
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "tok_per_s": round(args.steps / wall, 1),
+        "tok_per_s_scope": "the timed step: the weight products of one token; decode_tok_per_s_end_to_end is a whole greedy decode",
         "roofline": {"bound": "hbm", "kernel": "gemv_q4k_kernel", "achieved": round(q4k_gbs, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(q4k_gbs / HBM_PEAK_GBS, 4),
                      "traffic": round(Q4K_TRAFFIC_OVER_ALGORITHMIC * q4k_bytes / n_launch),
@@ -405,7 +408,15 @@ def main():
         out["other_workloads"] = other_workloads(pkg, hip, gpu, stream, rng, args.cpu_seconds > 0)
     if args.e2e_layers > 0:
         log("[bench] end-to-end greedy decode ...")
-        out.setdefault("other_workloads", {})["llama_greedy_decode"] = greedy_decode(pkg, args.e2e_layers, args.e2e_check, args.seed)
+        e2e = greedy_decode(pkg, args.e2e_layers, args.e2e_check, args.seed)
+        out.setdefault("other_workloads", {})["llama_greedy_decode"] = e2e
+        if args.e2e_layers == N_LAYERS:
+            # whole tokens per second of a real greedy decode (attention, norms and sampling included): the
+            # step resident on the GPU, and through the reference's host seam (one round trip per product)
+            out["decode_tok_per_s_end_to_end"] = e2e["device_session"]["decode_tok_per_s"]
+            out["decode_tok_per_s_host_seam"] = e2e["decode_tok_per_s"]
+            out["greedy_tokens_identical_to_cpu_path"] = bool(e2e.get("tokens_identical")) and bool(
+                e2e["device_session"].get("tokens_identical_to_cpu_path")) if args.e2e_check else None
     if args.cpu_seconds > 0:
         log("[bench] timing the CPU baseline ...")
         out["cpu_baseline"] = cpu_baseline(sample, x_host, args.cpu_seconds)
