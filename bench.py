@@ -43,7 +43,7 @@ BF16_MFMA_PEAK_TFLOPS = 2500.0
 # HBM bytes per Q4_K launch over algorithmic bytes, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this script (counters scaled by a 1 GiB copy kernel: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the
 # figures and commands are in profiles/decode_gemv_q4k_q6k_8b_step.txt.  Not measured by this run.
-Q4K_TRAFFIC_OVER_ALGORITHMIC = 1.0118
+Q4K_TRAFFIC_OVER_ALGORITHMIC = 1.0089
 Q4_0, Q8_0, Q4_K, Q6_K = 2, 8, 12, 14
 BLOCK = {Q4_0: (32, 18, 0), Q8_0: (32, 34, 0), Q4_K: (256, 144, 0), Q6_K: (256, 210, 208)}  # columns, bytes, offset of d
 N_LAYERS, D, D_KV, FF, VOCAB = 32, 4096, 1024, 14336, 128256
