@@ -44,8 +44,9 @@ BF16_MFMA_PEAK_TFLOPS = 2500.0
 # this script (counters scaled by a 1 GiB copy kernel: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the
 # figures and commands are in profiles/decode_gemv_q4k_q6k_8b_step.txt.  Not measured by this run.
 Q4K_TRAFFIC_OVER_ALGORITHMIC = 1.0089
-Q4_0, Q8_0, Q4_K, Q6_K = 2, 8, 12, 14
-BLOCK = {Q4_0: (32, 18, 0), Q8_0: (32, 34, 0), Q4_K: (256, 144, 0), Q6_K: (256, 210, 208)}  # columns, bytes, offset of d
+Q4_0, Q5_0, Q5_1, Q8_0, Q4_K, Q6_K = 2, 6, 7, 8, 12, 14
+BLOCK = {Q4_0: (32, 18, 0), Q5_0: (32, 22, 0), Q5_1: (32, 24, 0), Q8_0: (32, 34, 0), Q4_K: (256, 144, 0),
+         Q6_K: (256, 210, 208)}  # columns, bytes, offset of d
 N_LAYERS, D, D_KV, FF, VOCAB = 32, 4096, 1024, 14336, 128256
 # (name, rows, cols, which activation buffer it reads).  Products that read the same buffer are
 # independent of each other (q/k/v of the normed hidden state, gate/up of the normed residual);
@@ -75,7 +76,7 @@ def synth_matrix(ty, rows, cols, rng):
     qk, bb, d_off = BLOCK[ty]
     nb = cols // qk
     blk = rng.integers(0, 256, size=(rows, nb, bb), dtype=np.uint8)
-    n_scales = 2 if ty == Q4_K else 1  # Q4_K: d and dmin
+    n_scales = 2 if ty in (Q4_K, Q5_1) else 1  # Q4_K: d and dmin; Q5_1: d and m
     blk[:, :, d_off:d_off + 2 * n_scales] = (np.abs(rng.normal(0, 0.02, (rows, nb, n_scales))).astype(np.float16)
                                              .view(np.uint8).reshape(rows, nb, 2 * n_scales))
     return blk.reshape(-1)
@@ -165,25 +166,35 @@ def other_workloads(pkg, hip, gpu, stream, rng, cpu):
     for m in ms:
         m.close()
 
-    # Q4_0 4096x14336 at 8..512 tokens (chunked prefill)
-    n = 8
-    ws = [synth_matrix(Q4_0, D, FF, rng) for _ in range(n)]
-    ms = [gpu.upload_packed(Q4_0, D, FF, w) for w in ws]
-    x = rng.normal(0, 1, 512 * FF).astype(np.float32)
-    xd, yd = hip.DeviceBuffer.from_numpy(x), hip.DeviceBuffer(512 * D * 4)
-    for tokens in (8, 32, 128, 512):
-        us = timed_us(hip, stream, lambda i: gpu.gemm_device(ms[i], tokens, xd.ptr, yd.ptr, stream.ptr), n, 5)
-        gpu.gemm_device(ms[0], tokens, xd.ptr, yd.ptr, stream.ptr); stream.synchronize()
-        check(f"Q4_0 GEMM M={tokens}", Q4_0, D, FF, tokens, ws[0], x[:tokens * FF], yd)
-        flops = 2.0 * D * FF * tokens
-        # three bf16 MFMA products per multiply-add (the f32 activations are split in three)
-        out[f"gemm_q4_0_4096x14336_m{tokens}"] = {
-            "call_us": round(us, 2), "tflops": round(flops / us / 1e6, 1),
-            "mfma_frac": round(3 * flops / us / 1e6 / BF16_MFMA_PEAK_TFLOPS, 4),
-            "weight_gbs": round(D * row_bytes(Q4_0, FF) / us / 1e3, 1), "bound": "mfma" if tokens >= 128 else "hbm",
-            "cpu_us": cpu_us(Q4_0, D, FF, tokens, ws[0], x[:tokens * FF], 256 if tokens >= 128 else D)}
-    for m in ms:
-        m.close()
+    # Q4_0 / Q5_0 / Q5_1, 4096x14336 (ffn_down) and 14336x4096 (gate/up), 1..512 tokens (continuous batching:
+    # decode tokens and prefill chunks in one product); eight matrices per shape so that no call is served
+    # from the 256 MB Infinity Cache
+    names = {Q4_0: "q4_0", Q5_0: "q5_0", Q5_1: "q5_1"}
+    for ty in (Q4_0, Q5_0, Q5_1):
+        for rows, cols in ((D, FF), (FF, D)):
+            n = 8
+            ws = [synth_matrix(ty, rows, cols, rng) for _ in range(n)]
+            ms = [gpu.upload_packed(ty, rows, cols, w) for w in ws]
+            x = rng.normal(0, 1, 512 * cols).astype(np.float32)
+            xd, yd = hip.DeviceBuffer.from_numpy(x), hip.DeviceBuffer(512 * rows * 4)
+            for tokens in (1, 8, 32, 128, 512):
+                us = timed_us(hip, stream, lambda i: gpu.gemm_device(ms[i], tokens, xd.ptr, yd.ptr, stream.ptr), n, 5)
+                gpu.gemm_device(ms[0], tokens, xd.ptr, yd.ptr, stream.ptr); stream.synchronize()
+                check(f"{names[ty]} GEMM {rows}x{cols} M={tokens}", ty, rows, cols, tokens, ws[0], x[:tokens * cols], yd)
+                flops = 2.0 * rows * cols * tokens
+                with_cpu = ty == Q4_0 and rows == D and tokens > 1
+                # three bf16 MFMA products per multiply-add (the f32 activations are split in three)
+                out[f"gemm_{names[ty]}_{rows}x{cols}_m{tokens}"] = {
+                    "call_us": round(us, 2), "tflops": round(flops / us / 1e6, 1),
+                    "mfma_frac": round(3 * flops / us / 1e6 / BF16_MFMA_PEAK_TFLOPS, 4) if tokens > 1 else None,
+                    "weight_gbs": round(rows * row_bytes(ty, cols) / us / 1e3, 1),
+                    "hbm_frac": round(algorithmic_bytes(ty, rows, cols, tokens) / us / 1e3 / HBM_PEAK_GBS, 4),
+                    "bound": "mfma" if tokens >= 128 else "hbm",
+                    "cpu_us": cpu_us(ty, rows, cols, tokens, ws[0], x[:tokens * cols], 256 if tokens >= 128 else rows)
+                    if with_cpu else None}
+            for m in ms:
+                m.close()
+            xd.free(); yd.free()
 
     # one MoE projection: 8 Q4_K experts 4096 -> 14336, 16 tokens each, one grouped call
     n_exp, per = 8, 16
@@ -203,6 +214,48 @@ def other_workloads(pkg, hip, gpu, stream, rng, cpu):
     for ms_ in ms:
         for m in ms_:
             m.close()
+
+    # A whole MoE feed-forward, Mixtral-shaped: 8 experts, top-2 of 64 tokens by softmax of N(0,1) router
+    # logits (ties to the lower index), tokens of an expert grouped; gate, up and down as one grouped call each
+    n_tok = 64
+    logits = rng.normal(0, 1, (n_tok, n_exp)).astype(np.float32)
+    order = np.argsort(-logits, axis=1, kind="stable")[:, :2]
+    counts = [int(np.sum(order == e)) for e in range(n_exp)]
+    pairs = sum(counts)
+    sets = 2  # 2 x 793 MB of expert weights
+    wg = [[synth_matrix(Q4_K, FF, D, rng) for _ in range(n_exp)] for _ in range(sets)]
+    wd = [[synth_matrix(Q4_K, D, FF, rng) for _ in range(n_exp)] for _ in range(sets)]
+    mg = [[gpu.upload_packed(Q4_K, FF, D, w) for w in ws_] for ws_ in wg]
+    mu = [[gpu.upload_packed(Q4_K, FF, D, w) for w in ws_] for ws_ in wg]   # same bytes, separate residency
+    md = [[gpu.upload_packed(Q4_K, D, FF, w) for w in ws_] for ws_ in wd]
+    x = rng.normal(0, 1, pairs * D).astype(np.float32)
+    h = rng.normal(0, 1, pairs * FF).astype(np.float32)
+    xd, hd_ = hip.DeviceBuffer.from_numpy(x), hip.DeviceBuffer.from_numpy(h)
+    gd, ud, yd2 = hip.DeviceBuffer(pairs * FF * 4), hip.DeviceBuffer(pairs * FF * 4), hip.DeviceBuffer(pairs * D * 4)
+
+    def layer(i):
+        gpu.gemm_grouped_device(mg[i], counts, xd.ptr, gd.ptr, stream.ptr)
+        gpu.gemm_grouped_device(mu[i], counts, xd.ptr, ud.ptr, stream.ptr)
+        gpu.gemm_grouped_device(md[i], counts, hd_.ptr, yd2.ptr, stream.ptr)
+
+    us = timed_us(hip, stream, layer, sets, 5)
+    layer(0); stream.synchronize()
+    e0 = next(e for e in range(n_exp) if counts[e] > 0)
+    off = sum(counts[:e0])
+    got = yd2.to_numpy(np.float32)[off * D:(off + counts[e0]) * D].reshape(counts[e0], D)[:, :32]
+    want = np.asarray(O.gemm_f64(Q4_K, FF, counts[e0], wd[0][e0][:32 * row_bytes(Q4_K, FF)],
+                                 h[off * FF:(off + counts[e0]) * FF], 32)).reshape(counts[e0], 32)
+    if not np.allclose(got, want, rtol=1e-4, atol=1e-4 * float(np.sqrt(np.mean(want ** 2)))):
+        raise RuntimeError("MoE layer: GPU output disagrees with the CPU oracle")
+    wbytes = n_exp * (2 * FF * row_bytes(Q4_K, D) + D * row_bytes(Q4_K, FF))
+    out["moe_layer_q4_k_8_experts_top2_64_tokens"] = {
+        "call_us": round(us, 2), "calls": 3, "tokens_per_expert": counts, "weight_gbs": round(wbytes / us / 1e3, 1),
+        "frac": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4), "tflops": round(2.0 * pairs * 3 * FF * D / us / 1e6, 1),
+        "bound": "hbm"}
+    for group in (mg, mu, md):
+        for ms_ in group:
+            for m in ms_:
+                m.close()
     return out
 
 
