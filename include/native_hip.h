@@ -158,6 +158,14 @@ enum { LNH_PROLOGUE_NONE = 0, LNH_PROLOGUE_RMSNORM = 1, LNH_PROLOGUE_SWIGLU = 2 
 int lnh_gemv_fused_device(lnh_exec *exec, size_t n_mats, const lnh_matrix *const *mats, const float *device_x,
                           float *const *device_ys, int accumulate, int prologue, const float *device_x2, float eps,
                           void *stream);
+/* device_h = SiLU(gate x') * (up x'), x' = device_x or, with LNH_PROLOGUE_RMSNORM, its RMSNorm times
+ * device_x2: the gate and up products of one launch (langtax/src/decode.rs:2968-2979) and the element-wise
+ * step that follows them (decode.rs:2981-2984, 11826-11830) in the launch's epilogue, so that neither gate
+ * nor up is written out.  LNH_ERR_UNSUPPORTED (nothing launched) unless both are Q4_K of one shape with
+ * rows of 2048 to 16384 columns and the launch gives every 256-column unit its own wavefront (up to about
+ * 67 M weights per matrix on this part): the caller then uses lnh_gemv_fused_device. */
+int lnh_gemv_swiglu_device(lnh_exec *exec, const lnh_matrix *gate, const lnh_matrix *up, const float *device_x,
+                           float *device_h, int prologue, const float *device_x2, float eps, void *stream);
 /* Measurement aid, no counterpart in the reference: a plain device-to-device copy kernel
  * (nbytes a multiple of 16) whose known traffic calibrates HBM byte counters. */
 int lnh_calibration_copy(lnh_exec *exec, void *device_dst, const void *device_src, size_t nbytes, void *stream);

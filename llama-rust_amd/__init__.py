@@ -107,6 +107,7 @@ def load_library():
         "lnh_gemm_batch_device": (C.c_int, [vp, sz, pvp, psz, pvp, pvp, vp]),
         "lnh_gemv_shared_device": (C.c_int, [vp, sz, pvp, vp, pvp, C.c_int, vp]),
         "lnh_gemv_fused_device": (C.c_int, [vp, sz, pvp, vp, pvp, C.c_int, C.c_int, vp, C.c_float, vp]),
+        "lnh_gemv_swiglu_device": (C.c_int, [vp, vp, vp, vp, vp, C.c_int, vp, C.c_float, vp]),
         "lnh_calibration_copy": (C.c_int, [vp, vp, vp, sz, vp]),
         "lnh_synchronize": (C.c_int, [vp]),
         "lnh_shape_checked": (C.c_int, [sz, sz, sz, sz, C.POINTER(u32), C.POINTER(u32)]),
@@ -343,6 +344,11 @@ class HipGemv:
         ys = (C.c_void_p * n)(*y_ptrs)
         self._check(self._lib.lnh_gemv_fused_device(self._h, n, mats, C.c_void_p(x_ptr), ys, int(accumulate), prologue,
                                                     C.c_void_p(x2_ptr), eps, C.c_void_p(stream)))
+
+    def gemv_swiglu_device(self, gate, up, x_ptr, h_ptr, prologue=PROLOGUE_NONE, x2_ptr=0, eps=0.0, stream=0):
+        """h = SiLU(gate x') * (up x') in one launch; x' = x or RMSNorm(x) * x2."""
+        self._check(self._lib.lnh_gemv_swiglu_device(self._h, gate._h, up._h, C.c_void_p(x_ptr), C.c_void_p(h_ptr),
+                                                     prologue, C.c_void_p(x2_ptr), eps, C.c_void_p(stream)))
 
     def calibration_copy(self, dst_ptr, src_ptr, nbytes, stream=0):
         self._check(self._lib.lnh_calibration_copy(self._h, C.c_void_p(dst_ptr), C.c_void_p(src_ptr), nbytes,

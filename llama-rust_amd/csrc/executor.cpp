@@ -581,6 +581,28 @@ int lnh_gemv_fused_device(lnh_exec *e, size_t n_mats, const lnh_matrix *const *m
     return gemv_shared_device(e, n_mats, mats, dx, dys, accumulate, prologue, dx2, eps, stream);
 }
 
+int lnh_gemv_swiglu_device(lnh_exec *e, const lnh_matrix *gate, const lnh_matrix *up, const float *dx, float *dh,
+                           int prologue, const float *dx2, float eps, void *stream) {
+    if (!e) return LNH_ERR_INVALID;
+    if (!dx || !dh) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    if (prologue != LNH_PROLOGUE_NONE && prologue != LNH_PROLOGUE_RMSNORM) return fail(e, LNH_ERR_INVALID, "unknown prologue");
+    if (prologue != LNH_PROLOGUE_NONE && !dx2) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    size_t inputs, outputs;
+    int rc = check_gemm(e, gate, 1, false, 0, 0, &inputs, &outputs);
+    if (rc == LNH_OK) rc = check_gemm(e, up, 1, false, 0, 0, &inputs, &outputs);
+    if (rc != LNH_OK) return rc;
+    if (gate->view.type != up->view.type || gate->view.cols != up->view.cols || gate->view.rows != up->view.rows)
+        return fail(e, LNH_ERR_INVALID, "gate and up must share dtype and shape");
+    hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
+    const hipError_t h = nh::launch_gemv_swiglu_pair(s, gate->view, up->view, dx, dh, prologue, dx2, eps);
+    if (h == hipErrorInvalidValue) {
+        (void)hipGetLastError();
+        return fail(e, LNH_ERR_UNSUPPORTED, "no paired SiLU*up epilogue for this dtype or shape");
+    }
+    if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
+    return LNH_OK;
+}
+
 int lnh_calibration_copy(lnh_exec *e, void *device_dst, const void *device_src, size_t nbytes, void *stream) {
     if (!e) return LNH_ERR_INVALID;
     if (!device_dst || !device_src || nbytes % 16 != 0) return fail(e, LNH_ERR_INVALID, "copy needs device pointers and a multiple of 16 bytes");

@@ -46,6 +46,12 @@ hipError_t launch_gemv_multi(hipStream_t stream, const MatView *mats, float *con
 hipError_t launch_gemv_multi_prologue(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x,
                                       bool accumulate, int prologue, const float *x2, float eps);
 
+// h = SiLU(gate x') * (up x'), x' = x or, with prologue 1, RMSNorm(x) * x2: the two products of one launch
+// combined in its epilogue (Q4_K matrices of equal shape whose launch gives every unit its own wavefront;
+// hipErrorInvalidValue otherwise, nothing launched).
+hipError_t launch_gemv_swiglu_pair(hipStream_t stream, const MatView &gate, const MatView &up, const float *x, float *h,
+                                   int prologue, const float *x2, float eps);
+
 // dst[0, nbytes) = src[0, nbytes) (nbytes a multiple of 16): reference traffic for counter calibration.
 hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t nbytes);
 

@@ -62,6 +62,7 @@ static hipError_t launch_gemv_t(hipStream_t stream, const MatView *mats, float *
     b.accumulate = accumulate;
     b.x2 = nullptr;
     b.eps = 0.f;
+    b.pair = 0;
     const size_t lds = ((size_t)b.x_pad + (T == T_F32 || T == T_F16 ? 0 : 2 * (size_t)b.n_chunks)) * sizeof(float);
     if (lds > g_lds_limit) return hipErrorInvalidValue;
     auto kern = gemv_kernel<T, R>;
@@ -157,14 +158,21 @@ static hipError_t launch_q4k_lb(hipStream_t stream, const GemvBatch &b, uint32_t
     const uint32_t needed = (units + NW - 1) / NW;
     if (grid > needed) grid = needed;
     const bool one = grid == needed;  // a wavefront for every unit
-    void (*kern)(GemvBatch, float);
-    if constexpr (PRO == PRO_NONE)
+    void (*kern)(GemvBatch, float) = nullptr;
+    if (b.pair) {
+        // the pair epilogue exists where a wavefront holds at most four rows, for one unit per wavefront
+        if constexpr (LB >= 16 && PRO != PRO_SWIGLU) {
+            if (one && fp8) kern = gemv_q4k_kernel<LB, NW, true, PL, true, PRO, true>;
+        }
+        if (!kern) return hipErrorInvalidValue;
+    } else if constexpr (PRO == PRO_NONE) {
         kern = fp8 ? (one ? gemv_q4k_kernel<LB, NW, true, PL, true> : gemv_q4k_kernel<LB, NW, true, PL, false>)
                    : (one ? gemv_q4k_kernel<LB, NW, false, PL, true> : gemv_q4k_kernel<LB, NW, false, PL, false>);
-    else
+    } else {
         kern = one ? gemv_q4k_kernel<LB, NW, true, PL, true, PRO> : gemv_q4k_kernel<LB, NW, true, PL, false, PRO>;
-    static size_t configured[4] = {0, 0, 0, 0};
-    size_t &conf = configured[2 * fp8 + one];
+    }
+    static size_t configured[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    size_t &conf = configured[4 * (b.pair != 0) + 2 * fp8 + one];
     if (lds > 48 * 1024 && lds > conf) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)g_lds_limit);
@@ -182,7 +190,7 @@ static uint32_t fill_unit_jobs(GemvBatch &b, const MatView *mats, float *const *
     b.x = x;
     b.x2 = nullptr;
     b.eps = 0.f;
-    b.pad2 = 0;
+    b.pair = 0;
     b.n_jobs = n_jobs;
     b.n_chunks = 0;
     b.x_pad = mats[0].cols;
@@ -213,6 +221,7 @@ struct GemvPrologue {
     int kind = PRO_NONE;        // PRO_RMSNORM: x2 = norm weights; PRO_SWIGLU: x2 = the up vector (x is gate)
     const float *x2 = nullptr;
     float eps = 0.f;
+    bool pair = false;          // two jobs (gate, up): y of the first receives SiLU(gate) * up
 };
 
 template <int PRO>
@@ -222,6 +231,7 @@ static hipError_t launch_gemv_q4k_pro(hipStream_t stream, const MatView *mats, f
     // one lane per super-block, at most 64 per row and launch: longer rows take several launches
     const UnitWindows win(nb, 64);
     if (PRO != PRO_NONE && win.n != 1) return hipErrorInvalidValue;  // a prologue needs all of x in one workgroup
+    if (pro.pair && (win.n != 1 || n_jobs != 2 || mats[0].rows != mats[1].rows)) return hipErrorInvalidValue;
     for (uint32_t w = 0; w < win.n; w++) {
         const uint32_t units = win.count(w, nb);
         uint32_t lbb = 1;  // super-blocks per row, rounded up to a power of two
@@ -239,6 +249,7 @@ static hipError_t launch_gemv_q4k_pro(hipStream_t stream, const MatView *mats, f
         b.accumulate = accumulate || w > 0;
         b.x2 = pro.x2;
         b.eps = pro.eps;
+        b.pair = pro.pair ? 1u : 0u;
         // x slots, the sub-block sums of x, and room for one partial sum per wavefront (RMSNorm prologue)
         const size_t lds = (size_t)(64 * (lbb * 4 + 4) + lbb * 8 + 16) * sizeof(float);
         if (lds > g_lds_limit) return hipErrorInvalidValue;
@@ -657,6 +668,21 @@ hipError_t launch_gemv_multi_prologue(hipStream_t stream, const MatView *mats, f
     pro.x2 = x2;
     pro.eps = eps;
     return launch_gemv_q4k(stream, mats, ys, n, x, accumulate, pro);
+}
+
+hipError_t launch_gemv_swiglu_pair(hipStream_t stream, const MatView &gate, const MatView &up, const float *x, float *h,
+                                   int prologue, const float *x2, float eps) {
+    if (gate.type != T_Q4_K || up.type != T_Q4_K || gate.cols != up.cols || gate.rows != up.rows || gate.rows == 0)
+        return hipErrorInvalidValue;
+    if (prologue != PRO_NONE && (prologue != PRO_RMSNORM || !x2)) return hipErrorInvalidValue;
+    const MatView mats[2] = {gate, up};
+    float *const ys[2] = {h, h};
+    GemvPrologue pro;
+    pro.kind = prologue;
+    pro.x2 = x2;
+    pro.eps = eps;
+    pro.pair = true;
+    return launch_gemv_q4k(stream, mats, ys, 2, x, false, pro);
 }
 
 hipError_t launch_gemm(hipStream_t stream, const MatView &m, const MatView &tiled, uint32_t tokens, const float *x,

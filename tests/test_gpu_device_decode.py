@@ -187,3 +187,65 @@ def test_fused_and_unfused_device_sessions_agree(pkg, llama, tmp_path, monkeypat
     monkeypatch.setenv("LLAMA_HIP_DECODE_UNFUSED", "1")
     tb, _, _ = m.session(device_positions=48).generate_greedy(prompt, 16)
     assert ta.tolist() == tb.tolist()
+
+
+@pytest.mark.parametrize("rows,cols,norm", [(14336, 4096, True), (14336, 4096, False), (1536, 2048, True), (1000, 8192, False)])
+def test_paired_swiglu_epilogue_equals_the_separate_steps(pkg, rows, cols, norm):
+    """h = SiLU(gate x') * (up x') from one launch against float64 on the dequantized weights: each product
+    inside its own f32 summation bound, propagated through SiLU * up."""
+    import cases as K
+    hip = importlib.import_module("llama-rust_amd.hiprt")
+    rng = np.random.default_rng(rows + cols)
+    gpu = pkg.HipGemv(0)
+    wg = K.random_packed(K.Q4_K, rows, cols, rng, signed=False, scale=0.02)
+    wu = K.random_packed(K.Q4_K, rows, cols, rng, signed=False, scale=0.02)
+    mg, mu = gpu.upload_packed(K.Q4_K, rows, cols, wg), gpu.upload_packed(K.Q4_K, rows, cols, wu)
+    x = rng.normal(0, 1.0, cols).astype(np.float32)
+    g = (1 + rng.normal(0, 0.05, cols)).astype(np.float32)
+    eps = 1e-5
+    dx, dg, dh = _device(hip, x), _device(hip, g), hip.DeviceBuffer(4 * rows)
+    dh.fill_byte(0xff)
+    if norm:
+        gpu.gemv_swiglu_device(mg, mu, dx.ptr, dh.ptr, pkg.PROLOGUE_RMSNORM, dg.ptr, eps)
+        x64 = x.astype(np.float64)
+        xin = x64 / np.sqrt(np.mean(x64 * x64) + eps) * g.astype(np.float64)
+    else:
+        gpu.gemv_swiglu_device(mg, mu, dx.ptr, dh.ptr)
+        xin = x.astype(np.float64)
+    gpu.synchronize()
+    got = dh.to_numpy(np.float32).astype(np.float64)
+    a = oracle.dequant(K.Q4_K, cols, wg, rows).astype(np.float64) @ xin
+    b = oracle.dequant(K.Q4_K, cols, wu, rows).astype(np.float64) @ xin
+    _, mag_a = oracle.gemm_f64_mag(K.Q4_K, cols, 1, wg, xin.astype(np.float32), rows)
+    _, mag_b = oracle.gemm_f64_mag(K.Q4_K, cols, 1, wu, xin.astype(np.float32), rows)
+    slack = 16 * 2.0 ** -24
+    ea = K.single_kernel_bound(cols, mag_a.ravel()) + slack * mag_a.ravel()
+    eb = K.single_kernel_bound(cols, mag_b.ravel()) + slack * mag_b.ravel()
+    with np.errstate(over="ignore"):
+        sig = 1 / (1 + np.exp(-a))
+    silu, dsilu = a * sig, sig * (1 + a * (1 - sig))
+    want = silu * b
+    # first-order propagation of the two products' bounds, second-order term, and the roundings of SiLU * up itself
+    bound = np.abs(dsilu * b) * ea + np.abs(silu) * eb + 2 * ea * eb + 8 * 2.0 ** -24 * np.abs(want) + 1e-30
+    assert np.all(np.abs(got - want) <= bound), float(np.max(np.abs(got - want) / bound))
+    gpu.close()
+
+
+def test_paired_swiglu_is_refused_where_it_is_not_built(pkg):
+    import cases as K
+    hip = importlib.import_module("llama-rust_amd.hiprt")
+    rng = np.random.default_rng(9)
+    gpu = pkg.HipGemv(0)
+    # another dtype; a launch too large to give every unit its own wavefront; rows shorter than 2048 columns; unequal shapes
+    for ty, rows, cols, rows2, code in ((K.Q8_0, 64, 4096, 64, pkg.ERR_UNSUPPORTED), (K.Q4_K, 65536, 4096, 65536, pkg.ERR_UNSUPPORTED),
+                                        (K.Q4_K, 64, 512, 64, pkg.ERR_UNSUPPORTED), (K.Q4_K, 64, 4096, 128, pkg.ERR_INVALID)):
+        a = gpu.upload_packed(ty, rows, cols, K.random_packed(ty, rows, cols, rng, signed=False, scale=0.02))
+        b = gpu.upload_packed(ty, rows2, cols, K.random_packed(ty, rows2, cols, rng, signed=False, scale=0.02))
+        dx, dh = _device(hip, np.ones(cols)), hip.DeviceBuffer(4 * rows)
+        dh.fill_byte(0x5a)
+        with pytest.raises(pkg.NativeHipError) as ei:
+            gpu.gemv_swiglu_device(a, b, dx.ptr, dh.ptr)
+        assert ei.value.code == code
+        gpu.synchronize()
+        assert set(dh.to_numpy(np.uint8).tolist()) == {0x5a}
+    gpu.close()
