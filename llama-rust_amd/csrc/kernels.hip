@@ -503,8 +503,13 @@ static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *co
 
 template <uint32_t T, int TT, int VQ, bool FB = false>
 static hipError_t launch_mm_main(hipStream_t stream, const MmBatch &b) {
+    // FB: the device's shortcut from nibbles to bf16 codes is usable (probed at start-up): the packed
+    // fp8 convert for Q4_K, the signed 4-bit convert for Q4_0
     if constexpr (T == T_Q4_K && !FB) {
         if (b.nibble_bf16) return launch_mm_main<T, TT, VQ, true>(stream, b);
+    }
+    if constexpr (T == T_Q4_0 && !FB) {
+        if (g_nibble_i4) return launch_mm_main<T, TT, VQ, true>(stream, b);
     }
     constexpr size_t lds = 2 * MmStage<T, TT>::BYTES;  // two pipeline stages
     auto kern = gemm_mfma_kernel<T, TT, VQ, FB>;
