@@ -537,9 +537,8 @@ static hipError_t launch_mm_t(hipStream_t stream, MmPlan &p, void *ws, size_t ws
             b.job[j].part = reinterpret_cast<float *>(part);
             part += up256((size_t)b.job[j].ksplit * b.job[j].tokens * b.job[j].m.rows * sizeof(float));
         }
-    const size_t split_threads = (size_t)p.n_groups * b.mpad;
-    hipLaunchKernelGGL(mm_xsplit_kernel<T>, dim3((unsigned)((split_threads + 255) / 256)), dim3(256), 0, stream, b,
-                       p.n_groups);
+    hipLaunchKernelGGL(mm_xsplit_kernel<T>, dim3((b.mpad + XS_TOK - 1) / XS_TOK, (p.n_groups + XS_GRP - 1) / XS_GRP),
+                       dim3(256), 0, stream, b, p.n_groups);
     hipError_t e;
     if (p.tt == 2) e = launch_mm_main<T, 2, 4>(stream, b);
     else if (p.max_tok <= 8) e = launch_mm_main<T, 1, 1>(stream, b);
