@@ -439,6 +439,7 @@ static bool mm_type(uint32_t type) { return type != T_F32 && type != T_F16 && ty
 struct MmPlan {
     MmBatch b;
     int tt;             // token tiles of 32 per workgroup (1 or 2)
+    bool tile16;        // 16-token tiles (gemm_mfma16_kernel) instead
     uint32_t max_tok;   // most tokens of any job
     uint32_t n_groups;  // groups of 16 columns
     size_t xb_bytes, sx_bytes, part_bytes;
@@ -454,7 +455,8 @@ static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *co
     for (uint32_t j = 0; j < n; j++) max_tok = tokens[j] > max_tok ? tokens[j] : max_tok;
     p.tt = max_tok > 32 ? 2 : 1;
     p.max_tok = max_tok;
-    const uint32_t tile_tok = 32u * (uint32_t)p.tt;
+    p.tile16 = max_tok <= 16 && mats[0].type != T_Q6_K;
+    const uint32_t tile_tok = p.tile16 ? 16u : 32u * (uint32_t)p.tt;
     uint32_t wgs = 0;
     bool any_split = false;
     const uint32_t n_steps = mats[0].cols / 32;
@@ -524,6 +526,19 @@ static hipError_t launch_mm_main(hipStream_t stream, const MmBatch &b) {
     return hipGetLastError();
 }
 
+template <uint32_t T, bool FB = false>
+static hipError_t launch_mm16_main(hipStream_t stream, const MmBatch &b) {
+    if constexpr (T == T_Q4_K && !FB) {
+        if (b.nibble_bf16) return launch_mm16_main<T, true>(stream, b);
+    }
+    if constexpr (T == T_Q4_0 && !FB) {
+        if (g_nibble_i4) return launch_mm16_main<T, true>(stream, b);
+    }
+    constexpr size_t lds = 2 * Mm16Traits<T>::BYTES;  // two pipeline stages
+    hipLaunchKernelGGL((gemm_mfma16_kernel<T, FB>), dim3(b.total_wgs), dim3(256), lds, stream, b);
+    return hipGetLastError();
+}
+
 template <uint32_t T>
 static hipError_t launch_mm_t(hipStream_t stream, MmPlan &p, void *ws, size_t ws_bytes) {
     if (p.xb_bytes + p.sx_bytes + p.part_bytes > ws_bytes) return hipErrorInvalidValue;
@@ -540,6 +555,14 @@ static hipError_t launch_mm_t(hipStream_t stream, MmPlan &p, void *ws, size_t ws
     hipLaunchKernelGGL(mm_xsplit_kernel<T>, dim3((b.mpad + XS_TOK - 1) / XS_TOK, (p.n_groups + XS_GRP - 1) / XS_GRP),
                        dim3(256), 0, stream, b, p.n_groups);
     hipError_t e;
+    if constexpr (T != T_Q6_K) {
+        if (p.tile16) {
+            e = launch_mm16_main<T>(stream, b);
+            if (e != hipSuccess) return e;
+            if (b.any_split) hipLaunchKernelGGL(mm_reduce_kernel, dim3(512, b.n_jobs), dim3(256), 0, stream, b);
+            return hipGetLastError();
+        }
+    }
     if (p.tt == 2) e = launch_mm_main<T, 2, 4>(stream, b);
     else if (p.max_tok <= 8) e = launch_mm_main<T, 1, 1>(stream, b);
     else if (p.max_tok <= 16) e = launch_mm_main<T, 1, 2>(stream, b);
