@@ -465,7 +465,7 @@ static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *co
     uint32_t launch_tiles = 0;
     for (uint32_t j = 0; j < n; j++)
         launch_tiles += ((tokens[j] + tile_tok - 1) / tile_tok) * ((mats[j].rows + MM_ROWS - 1) / MM_ROWS);
-    uint32_t ks_launch = (uint32_t)(2 * g_cu_count) / (launch_tiles ? launch_tiles : 1);  // two workgroups per CU (measured best of 1..4)
+    uint32_t ks_launch = (uint32_t)(2 * g_cu_count) / (launch_tiles ? launch_tiles : 1);  // two workgroups per CU (measured best of 1..4, both tile sizes)
     if (ks_launch > n_steps / 8) ks_launch = n_steps / 8;                                 // shares are whole 256-column units
     if (ks_launch > 32) ks_launch = 32;
     if (ks_launch < 1) ks_launch = 1;
@@ -619,16 +619,43 @@ static uint32_t mm_run(const MatView *mats, const uint32_t *tokens, uint32_t n, 
     return run;
 }
 
+// A run is launched as up to two batches: the products of at most 16 tokens (16-token tiles) and the
+// others (32- or 64-token tiles); a product of 9 tokens beside one of 21 would otherwise pay for 32.
+struct MmClass {
+    MatView mats[MM_MAX_JOBS];
+    uint32_t tokens[MM_MAX_JOBS];
+    const float *xs[MM_MAX_JOBS];
+    float *ys[MM_MAX_JOBS];
+    uint32_t n;
+};
+static void mm_classes(const MatView *mats, const uint32_t *tokens, const float *const *xs, float *const *ys, uint32_t run,
+                       MmClass (&cls)[2]) {
+    cls[0].n = cls[1].n = 0;
+    for (uint32_t j = 0; j < run; j++) {
+        MmClass &c = cls[tokens[j] <= 16 && mats[j].type != T_Q6_K ? 0 : 1];
+        c.mats[c.n] = mats[j];
+        c.tokens[c.n] = tokens[j];
+        c.xs[c.n] = xs ? xs[j] : nullptr;
+        c.ys[c.n] = ys ? ys[j] : nullptr;
+        c.n++;
+    }
+}
+
 size_t gemm_workspace_bytes(const MatView *mats, const uint32_t *tokens, uint32_t n) {
     size_t need = 0;
     for (uint32_t g = 0; g < n;) {
         if (tokens[g] == 0 || mats[g].rows == 0) { g++; continue; }
         const uint32_t run = mm_run(mats, tokens, n, g);
         if (run == 0) { g++; continue; }
-        MmPlan p;
-        mm_plan(mats + g, tokens + g, nullptr, nullptr, run, p);
-        const size_t bytes = p.xb_bytes + p.sx_bytes + p.part_bytes;
-        need = bytes > need ? bytes : need;
+        MmClass cls[2];
+        mm_classes(mats + g, tokens + g, nullptr, nullptr, run, cls);
+        for (const MmClass &c : cls) {
+            if (c.n == 0) continue;
+            MmPlan p;
+            mm_plan(c.mats, c.tokens, nullptr, nullptr, c.n, p);
+            const size_t bytes = p.xb_bytes + p.sx_bytes + p.part_bytes;
+            need = bytes > need ? bytes : need;
+        }
         g += run;
     }
     return need;
@@ -639,14 +666,19 @@ hipError_t launch_gemm_groups(hipStream_t stream, const MatView *mats, const Mat
     for (uint32_t g = 0; g < n;) {
         if (tokens[g] == 0 || mats[g].rows == 0) { g++; continue; }
         const uint32_t run = mm_run(mats, tokens, n, g);
-        hipError_t e;
+        hipError_t e = hipSuccess;
         if (run == 0) {
             e = launch_plain(stream, mats[g], tokens[g], xs[g], ys[g]);
             g++;
         } else {
-            MmPlan p;
-            mm_plan(tiled + g, tokens + g, xs + g, ys + g, run, p);
-            e = launch_mm(stream, p, ws, ws_bytes);
+            MmClass cls[2];
+            mm_classes(tiled + g, tokens + g, xs + g, ys + g, run, cls);
+            for (const MmClass &c : cls) {  // the batches follow each other on the stream and share the workspace
+                if (c.n == 0 || e != hipSuccess) continue;
+                MmPlan p;
+                mm_plan(c.mats, c.tokens, c.xs, c.ys, c.n, p);
+                e = launch_mm(stream, p, ws, ws_bytes);
+            }
             g += run;
         }
         if (e != hipSuccess) return e;
