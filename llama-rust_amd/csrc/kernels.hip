@@ -489,7 +489,7 @@ static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *co
     }
     for (uint32_t j = n; j < MM_MAX_JOBS; j++) b.job[j] = b.job[0];
     b.n_jobs = n;
-    b.mpad = total_tok + 64;  // a tile may read up to 63 slots past its job's last token
+    b.mpad = total_tok + (p.tile16 ? 16 : 64);  // a tile may read up to 15 resp. 63 slots past its job's last token
     b.total_wgs = wgs;
     b.any_split = any_split ? 1u : 0u;
     b.nibble_bf16 = g_nibble_bf16 ? 1u : 0u;
