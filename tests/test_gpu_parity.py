@@ -245,7 +245,7 @@ def test_random_gemv_and_gemm_within_bounds(pkg, gpu, ty):
     for rows, cols in shapes:
         w = K.random_packed(ty, rows, cols, rng)
         m = gpu.upload_packed(ty, rows, cols, w)
-        for tokens in (1, 2, 5, 8, 33):
+        for tokens in (1, 2, 5, 8, 13, 16, 17, 33):
             x = rng.normal(0, 1, tokens * cols).astype(np.float32)
             y = np.full(tokens * rows, np.nan, np.float32)
             gpu.gemm_resident(m, tokens, x, y)
