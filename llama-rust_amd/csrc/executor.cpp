@@ -40,6 +40,8 @@ struct lnh_exec {
     hipStream_t stream = nullptr;
     float *d_in = nullptr, *d_out = nullptr;  // device scratch, grow-only
     size_t in_cap = 0, out_cap = 0;           // capacities in floats
+    float *h_in = nullptr, *h_out = nullptr;  // pinned host staging for small calls, grow-only
+    size_t hin_cap = 0, hout_cap = 0;
     void *d_ws = nullptr;                     // kernel workspace (multi-token products), grow-only
     size_t ws_cap = 0;
     std::string err;
@@ -90,7 +92,7 @@ int ensure_scratch(lnh_exec *e, size_t in_floats, size_t out_floats) {
             buf = nullptr;
             cap = 0;
         }
-        size_t n = want < 4096 ? 4096 : want;
+        size_t n = want < 4096 ? 4096 : (want + 3) & ~(size_t)3;  // whole 16-byte vectors (launch_copy_small)
         hipError_t h = hipMalloc(reinterpret_cast<void **>(&buf), n * sizeof(float));
         if (h == hipSuccess) cap = n;
         return h;
@@ -107,6 +109,29 @@ int ensure_scratch(lnh_exec *e, size_t in_floats, size_t out_floats) {
         e->in_cap = e->out_cap = 0;
     }
     return LNH_ERR_OOM;
+}
+
+// Pinned host staging for calls whose activations are small (a decode step's vectors, a few tokens).
+// A copy from or to pageable memory makes the runtime stage and synchronise on its own, tens of
+// microseconds per call; from pinned memory a small kernel moves the data at PCIe latency.  False = no
+// pinned memory to be had: the caller takes the plain copies.
+constexpr size_t PINNED_MAX_FLOATS = (size_t)1 << 20;  // 4 MB each way
+bool ensure_pinned(lnh_exec *e, size_t in_floats, size_t out_floats) {
+    auto grow = [&](float *&buf, size_t &cap, size_t want) {
+        if (want <= cap) return true;
+        if (buf) (void)hipHostFree(buf);
+        buf = nullptr;
+        cap = 0;
+        size_t n = want < 16384 ? 16384 : (want + 3) & ~(size_t)3;
+        if (hipHostMalloc(reinterpret_cast<void **>(&buf), n * sizeof(float), hipHostMallocDefault) != hipSuccess) {
+            (void)hipGetLastError();
+            buf = nullptr;
+            return false;
+        }
+        cap = n;
+        return true;
+    };
+    return grow(e->h_in, e->hin_cap, in_floats) && grow(e->h_out, e->hout_cap, out_floats);
 }
 
 // Workspace of the multi-token kernels.  Work already queued that uses the old
@@ -248,7 +273,13 @@ int run_host(lnh_exec *e, size_t n_groups, const lnh_matrix *const *mats, const 
     if (h != hipSuccess) return hip_fail(e, h, "hipSetDevice");
     int rc = ensure_scratch(e, x_total, y_total);
     if (rc != LNH_OK) return rc;
-    h = hipMemcpyAsync(e->d_in, x, x_total * sizeof(float), hipMemcpyHostToDevice, e->stream);
+    const bool pinned = x_total <= PINNED_MAX_FLOATS && y_total <= PINNED_MAX_FLOATS && ensure_pinned(e, x_total, y_total);
+    if (pinned) {
+        std::memcpy(e->h_in, x, x_total * sizeof(float));
+        h = nh::launch_copy_small(e->stream, e->d_in, e->h_in, ((x_total + 3) & ~(size_t)3) * sizeof(float));
+    } else {
+        h = hipMemcpyAsync(e->d_in, x, x_total * sizeof(float), hipMemcpyHostToDevice, e->stream);
+    }
     if (h != hipSuccess) return hip_fail(e, h, "HIP input copy");
     std::vector<const float *> xs(n_groups);
     std::vector<float *> ys(n_groups);
@@ -264,10 +295,14 @@ int run_host(lnh_exec *e, size_t n_groups, const lnh_matrix *const *mats, const 
         (void)hipStreamSynchronize(e->stream);
         return rc;
     }
-    h = hipMemcpyAsync(y, e->d_out, y_total * sizeof(float), hipMemcpyDeviceToHost, e->stream);
+    if (pinned)
+        h = nh::launch_copy_small(e->stream, e->h_out, e->d_out, ((y_total + 3) & ~(size_t)3) * sizeof(float));
+    else
+        h = hipMemcpyAsync(y, e->d_out, y_total * sizeof(float), hipMemcpyDeviceToHost, e->stream);
     hipError_t hs = hipStreamSynchronize(e->stream);
     if (h == hipSuccess) h = hs;
     if (h != hipSuccess) return hip_fail(e, h, "HIP output copy");
+    if (pinned) std::memcpy(y, e->h_out, y_total * sizeof(float));  // y is written only after everything succeeded
     return LNH_OK;
 }
 
@@ -322,6 +357,8 @@ void lnh_destroy(lnh_exec *e) {
     if (e->d_ws) (void)hipFree(e->d_ws);
     if (e->d_in) (void)hipFree(e->d_in);
     if (e->d_out) (void)hipFree(e->d_out);
+    if (e->h_in) (void)hipHostFree(e->h_in);
+    if (e->h_out) (void)hipHostFree(e->h_out);
     delete e;
 }
 

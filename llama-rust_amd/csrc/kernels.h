@@ -54,5 +54,8 @@ hipError_t launch_gemv_swiglu_pair(hipStream_t stream, const MatView &gate, cons
 
 // dst[0, nbytes) = src[0, nbytes) (nbytes a multiple of 16): reference traffic for counter calibration.
 hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t nbytes);
+// The same copy with a grid sized by nbytes: activations between pinned host staging memory (which the
+// device reads and writes directly) and device scratch, a few KB at a time.
+hipError_t launch_copy_small(hipStream_t stream, void *dst, const void *src, size_t nbytes);
 
 }  // namespace nh

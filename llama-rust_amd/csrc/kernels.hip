@@ -697,6 +697,14 @@ hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t nb
     return hipGetLastError();
 }
 
+hipError_t launch_copy_small(hipStream_t stream, void *dst, const void *src, size_t nbytes) {
+    const size_t n16 = nbytes / 16, want = (n16 + 255) / 256, most = (size_t)g_cu_count * 8;
+    if (n16 == 0) return hipSuccess;
+    hipLaunchKernelGGL(copy_kernel, dim3((unsigned)(want < most ? want : most)), dim3(256), 0, stream,
+                       static_cast<uint4 *>(dst), static_cast<const uint4 *>(src), n16);
+    return hipGetLastError();
+}
+
 hipError_t launch_gemv_multi(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x,
                              bool accumulate) {
     if (n == 0) return hipSuccess;

@@ -280,14 +280,18 @@ def test_adversarial_activations_keep_the_reference_bound(pkg, gpu, ty):
     # token 5: one large value among small ones (cancellation in the other columns must survive)
     x[5] = rng.normal(0, 1e-3, cols).astype(np.float32)
     x[5, 777] = 3.0e4
-    y = np.full(tokens * rows, np.nan, np.float32)
-    gpu.gemm_resident(m, tokens, x.reshape(-1), y)
     exact, mag = O.gemm_f64_mag(ty, cols, tokens, w, x.reshape(-1), rows)
-    err = np.abs(y.reshape(tokens, rows).astype(np.float64) - exact)
-    assert np.all(np.isfinite(y))
-    # the reference's proven bound and its observed envelope, per output, relative to sum |w x|
-    assert np.all(err <= K.single_kernel_bound(cols, mag))
-    assert np.all(err <= K.observed_envelope_u(cols) * K.U * mag)
+    # 6 tokens run on the 16-token tiles, the same 6 three times over (18) on the 32-token tiles
+    for reps in (1, 3):
+        xr = np.tile(x, (reps, 1))
+        y = np.full(reps * tokens * rows, np.nan, np.float32)
+        gpu.gemm_resident(m, reps * tokens, xr.reshape(-1), y)
+        assert np.all(np.isfinite(y))
+        for rep in range(reps):
+            err = np.abs(y.reshape(reps, tokens, rows)[rep].astype(np.float64) - exact)
+            # the reference's proven bound and its observed envelope, per output, relative to sum |w x|
+            assert np.all(err <= K.single_kernel_bound(cols, mag)), f"{reps * tokens} tokens"
+            assert np.all(err <= K.observed_envelope_u(cols) * K.U * mag), f"{reps * tokens} tokens"
     # the single-token kernels on the same rows: the same bounds (a code bias factored out
     # through the sum of x would fail here: one large activation under a zero weight)
     for t in range(tokens):
