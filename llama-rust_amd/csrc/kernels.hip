@@ -610,10 +610,13 @@ static hipError_t launch_plain(hipStream_t stream, const MatView &m, uint32_t to
 }
 
 // Length of the run of groups starting at g that one MFMA launch can take.
+// (Two tokens are two single-token launches: 2 x 9-15 us on the 33-44 MB matrices against 24-29 us for the
+// three launches of the MFMA path, and row t of the result is then bit for bit the GEMV of token t.)
+constexpr uint32_t MM_MIN_TOKENS = 3;
 static uint32_t mm_run(const MatView *mats, const uint32_t *tokens, uint32_t n, uint32_t g) {
-    if (!mm_type(mats[g].type) || tokens[g] < 2) return 0;
+    if (!mm_type(mats[g].type) || tokens[g] < MM_MIN_TOKENS) return 0;
     uint32_t run = 1;
-    while (g + run < n && run < (uint32_t)MM_MAX_JOBS && tokens[g + run] >= 2 && mats[g + run].type == mats[g].type &&
+    while (g + run < n && run < (uint32_t)MM_MAX_JOBS && tokens[g + run] >= MM_MIN_TOKENS && mats[g + run].type == mats[g].type &&
            mats[g + run].cols == mats[g].cols)
         run++;
     return run;
@@ -668,7 +671,12 @@ hipError_t launch_gemm_groups(hipStream_t stream, const MatView *mats, const Mat
         const uint32_t run = mm_run(mats, tokens, n, g);
         hipError_t e = hipSuccess;
         if (run == 0) {
-            e = launch_plain(stream, mats[g], tokens[g], xs[g], ys[g]);
+            if (mm_type(mats[g].type) && tokens[g] > 1) {
+                for (uint32_t t = 0; t < tokens[g] && e == hipSuccess; t++)
+                    e = launch_plain(stream, mats[g], 1, xs[g] + (size_t)t * mats[g].cols, ys[g] + (size_t)t * mats[g].rows);
+            } else {
+                e = launch_plain(stream, mats[g], tokens[g], xs[g], ys[g]);
+            }
             g++;
         } else {
             MmClass cls[2];
