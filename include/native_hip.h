@@ -125,7 +125,7 @@ int lnh_gemm_shared(lnh_exec *exec, size_t n_mats, const lnh_matrix *const *mats
  * `stream` (a hipStream_t; NULL = the executor's own stream) without any host
  * synchronisation.  No counterpart in the reference, whose every call copies
  * through the host (native-cuda/src/gpu.rs:301-303, 332-334).
- * Products of two or more tokens by a quantized matrix use a workspace that
+ * Products of three or more tokens by a quantized matrix use a workspace that
  * belongs to the executor and grows on demand (growing allocates, so it cannot
  * happen while `stream` is being captured into a graph: run the largest shape
  * once before capturing).  Calls of one executor must therefore be enqueued on

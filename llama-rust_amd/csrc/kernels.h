@@ -21,7 +21,8 @@ hipError_t launch_repack(hipStream_t stream, const MatView &m, const void *src_d
 hipError_t launch_repack_tiled(hipStream_t stream, const MatView &tiled, const void *src_device);
 
 // y[t, r] = sum_c W[r, c] x[t, c]; x and y are device pointers, token-major.
-// Products of two or more tokens by a quantized matrix run on the matrix cores,
+// Products of three or more tokens by a quantized matrix run on the matrix cores (two tokens: two
+// single-token launches),
 // read the tiled copy of the matrix and need device workspace: ws must hold gemm_workspace_bytes() for the same
 // arguments (hipErrorInvalidValue otherwise).  The workspace is only used by
 // work queued on `stream`, so calls on one stream may share it.

@@ -447,7 +447,7 @@ struct MmPlan {
 
 static size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
 
-// Jobs share dtype and column count; every job has at least two tokens.
+// Jobs share dtype and column count; every job has at least MM_MIN_TOKENS tokens.
 static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *const *xs, float *const *ys, uint32_t n,
                     MmPlan &p) {
     MmBatch &b = p.b;
