@@ -294,7 +294,7 @@ def greedy_decode(pkg, layers, check_cpu, seed):
                                  "decode_s": round(dd, 4), "decode_tok_per_s": round(128 / dd, 1),
                                  "ms_per_token": round(dd / 128 * 1e3, 3),
                                  "tokens_identical_to_host_session": bool(dsame == 129), "identical_prefix": dsame}
-        log(f"[bench] device session: prompt token by token {dp:.2f} s, 128 steps in {dd:.3f} s ({128 / dd:.0f} tok/s)")
+        log(f"[bench] device session: prompt (127 tokens as one batch, the last as a step) {dp:.3f} s, 128 steps in {dd:.3f} s ({128 / dd:.0f} tok/s)")
         dev.close()
         m.close()
         if check_cpu:

@@ -189,6 +189,34 @@ def test_fused_and_unfused_device_sessions_agree(pkg, llama, tmp_path, monkeypat
     assert ta.tolist() == tb.tolist()
 
 
+@pytest.mark.parametrize("n_prompt", [3, 17, 140, 300])
+def test_prompt_as_batches_equals_prompt_step_by_step(pkg, llama, tmp_path, monkeypatch, n_prompt):
+    """All prompt tokens but the last run through the multi-token kernels in chunks of up to 128 (K and V into
+    the cache, nothing else kept); LLAMA_HIP_DECODE_STEP_PREFILL runs them as single steps like decode.  Same
+    tokens, logits to 1e-4, also across chunk boundaries (140: 128 + 11; 300: 128 + 128 + 43), for a prompt
+    continued by a second one in the same session, and against the host session."""
+    path = tmp_path / "small.gguf"
+    llama.write_synthetic_llama(path, n_layer=3, n_embd=512, n_head=8, n_head_kv=2, n_ff=1536, n_vocab=2048, seed=35)
+    m = llama.Llama(path=path)
+    rng = np.random.default_rng(n_prompt)
+    prompt = rng.integers(0, 2048, n_prompt).tolist()
+    more = rng.integers(0, 2048, 9).tolist()
+    cap = n_prompt + 9 + 12
+    batched = m.session(device_positions=cap)
+    monkeypatch.setenv("LLAMA_HIP_DECODE_STEP_PREFILL", "1")
+    stepped = m.session(device_positions=cap)
+    monkeypatch.delenv("LLAMA_HIP_DECODE_STEP_PREFILL")
+    host = m.session()
+    la, lb, lh = batched.forward(prompt), stepped.forward(prompt), host.forward(prompt)
+    assert logits_close(la, lb) and logits_close(la, lh)
+    la, lb, lh = batched.forward(more), stepped.forward(more), host.forward(more)  # a second chunk at past > 0
+    assert logits_close(la, lb) and logits_close(la, lh)
+    ta, _, _ = m.session(device_positions=cap).generate_greedy(prompt, 12)
+    monkeypatch.setenv("LLAMA_HIP_DECODE_STEP_PREFILL", "1")
+    tb, _, _ = m.session(device_positions=cap).generate_greedy(prompt, 12)
+    assert ta.tolist() == tb.tolist()
+
+
 @pytest.mark.parametrize("rows,cols,norm", [(14336, 4096, True), (14336, 4096, False), (1536, 2048, True), (1000, 8192, False)])
 def test_paired_swiglu_epilogue_equals_the_separate_steps(pkg, rows, cols, norm):
     """h = SiLU(gate x') * (up x') from one launch against float64 on the dequantized weights: each product
