@@ -71,7 +71,9 @@ int lnm_session_new(lnm_model *model, size_t kv_block, const uint32_t *block_ids
  * on in device memory.  No counterpart in the reference, whose every product returns to the host
  * (langtax/src/native_gpu.rs:124-213); the arithmetic of the small kernels is the host code's, element for
  * element, except for the order of the sums inside RMSNorm and the softmax denominator.
- * `max_positions` sizes the cache (rounded up to whole blocks); a batch of n tokens runs as n steps. */
+ * `max_positions` sizes the cache (rounded up to whole blocks).  A batch of n >= 3 tokens runs its first n - 1
+ * tokens through the multi-token products in chunks of up to 128 (only their K and V are kept) and the last one
+ * as a step; the environment variable LLAMA_HIP_DECODE_STEP_PREFILL makes every token a step. */
 int lnm_session_new_device(lnm_model *model, size_t kv_block, const uint32_t *block_ids, size_t n_block_ids,
                            size_t max_positions, lnm_session **out);
 void lnm_session_free(lnm_session *session);
