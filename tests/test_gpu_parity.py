@@ -477,6 +477,38 @@ def test_grouped_gemm_with_empty_groups_and_dispatch_layer(pkg):
         yo += t * rows
 
 
+@pytest.mark.parametrize("ty", [K.Q4_0, K.Q5_1, K.Q8_0, K.Q4_K, K.Q6_K], ids=lambda t: O.TYPE_NAMES[t])
+def test_grouped_call_with_token_counts_on_both_sides_of_every_kernel_switch(pkg, gpu, ty):
+    """One grouped call whose products have 0, 1, 2, 3, 16, 17, 33 and 70 tokens: single-token launches
+    (1 and 2), the 16-token tiles (3, 16; not Q6_K), the 32-token tiles (17) and the 64-token tiles (33, 70)
+    inside one call, in an order that interleaves the classes.  Every group against the oracle, and bit for
+    bit equal to the same product called on its own."""
+    rng = np.random.default_rng(77 + ty)
+    rows, cols = 160, 1024
+    tokens = [17, 3, 0, 70, 1, 16, 2, 33]
+    ws = [K.random_packed(ty, rows, cols, rng) for _ in tokens]
+    mats = [gpu.upload_packed(ty, rows, cols, w) for w in ws]
+    x = rng.normal(0, 1, sum(tokens) * cols).astype(np.float32)
+    y = np.full(sum(tokens) * rows, np.nan, np.float32)
+    gpu.gemm_grouped(mats, tokens, x, y)
+    xo = yo = 0
+    for g, t in enumerate(tokens):
+        if t:
+            yg, xg = y[yo:yo + t * rows], x[xo:xo + t * cols]
+            check(yg, ty, cols, t, rows, ws[g], xg, f"{O.TYPE_NAMES[ty]} group {g} M={t}")
+            alone = np.full(t * rows, np.nan, np.float32)
+            gpu.gemm_resident(mats[g], t, xg, alone)
+            if t <= 2:
+                assert np.array_equal(yg, alone)  # the same single-token launches
+            else:  # a launch shares out columns by its total size: the same products, another order of the f32 sums
+                rms = float(np.sqrt(np.mean(alone.astype(np.float64) ** 2)))
+                assert np.max(np.abs(yg.astype(np.float64) - alone)) <= 2e-5 * rms
+        xo += t * cols
+        yo += t * rows
+    for m in mats:
+        m.close()
+
+
 def test_shared_input_products_equal_separate_calls(pkg, gpu):
     """q, k, v (and gate, up) read the same activations: one call, one input copy.  The values are those
     of the separate calls bit for bit (same kernels, same order of additions within each row)."""
