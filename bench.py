@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the decode GEMV hot path on one MI355X.
 
-Workload (BASELINE config "Llama-3-8B decode layer shapes as batch-1 GEMV"): one
+Workload (benchmark configuration "Llama-3-8B decode layer shapes as batch-1 GEMV"): one
 step is one generated token's weight products, batch 1 - for each of 32 layers
 the seven Q4_K GEMVs q, k, v, o (4096->4096/1024), gate, up (4096->14336), down
 (14336->4096), then the Q6_K output head 4096->128256 - 225 products streaming
@@ -260,7 +260,7 @@ def other_workloads(pkg, hip, gpu, stream, rng, cpu):
 
 
 def greedy_decode(pkg, layers, check_cpu, seed):
-    """BASELINE config 4: a random Llama-3-8B-shaped Q4_K / Q6_K-head GGUF, 128 prompt ids as one
+    """Benchmark configuration 4: a random Llama-3-8B-shaped Q4_K / Q6_K-head GGUF, 128 prompt ids as one
     batch, then 128 greedy single-token steps through the host decode (host attention and norms,
     every weight product on the GPU with host round trips, as the reference's executor is called).
     With check_cpu the same host code runs again over the CPU kernels and the tokens are compared."""
@@ -326,7 +326,7 @@ def main():
     ap.add_argument("--seed", type=int, default=20240531)
     ap.add_argument("--no-extras", action="store_true", help="skip the other_workloads section")
     ap.add_argument("--e2e-layers", type=int, default=32,
-                    help="layers of the model of the end-to-end greedy decode (128 prompt + 128 steps); 32 = BASELINE config 4, 0 skips it")
+                    help="layers of the model of the end-to-end greedy decode (128 prompt + 128 steps); 32 = benchmark configuration 4, 0 skips it")
     ap.add_argument("--e2e-check", action="store_true", default=True,
                     help="repeat the greedy decode over the CPU kernels and compare tokens (default)")
     ap.add_argument("--no-e2e-check", dest="e2e_check", action="store_false")
@@ -335,7 +335,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         log(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); "
-            "the path shards by weight rows, which is described in DESIGN.md but not built")
+            "the path shards by weight rows, which is designed but not built")
         return 2
 
     pkg = importlib.import_module("llama-rust_amd")

@@ -1,7 +1,7 @@
 """Parity of the HIP executor with the CPU oracle, through the C ABI, on a real
 MI355X.  The cases restate the reference's own executor self-test
 (native-cuda/src/main.rs) and integration contract
-(langtax/tests/native_cuda_parity.rs) and add random data at the BASELINE
+(langtax/tests/native_cuda_parity.rs) and add random data at the benchmark
 shapes.
 
 Tolerances (floating point, f32 accumulation), all against an f64 product of the
@@ -330,9 +330,9 @@ def test_every_f16_scale_pattern_and_zero_blocks(pkg, gpu, ty):
     m.close()
 
 
-# ------------------------------------------------------------------ BASELINE shapes
+# ------------------------------------------------------------------ benchmark shapes
 def _baseline_matrix(ty, rows, cols, rng):
-    """Synthetic weights with BASELINE's distributions: |N(0, 0.02)| block scales, uniform codes."""
+    """Synthetic weights with the benchmark configurations' distributions: |N(0, 0.02)| block scales, uniform codes."""
     return K.random_packed(ty, rows, cols, rng, signed=False, scale=0.02)
 
 
