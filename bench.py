@@ -296,6 +296,19 @@ def greedy_decode(pkg, layers, check_cpu, seed):
                                  "tokens_identical_to_host_session": bool(dsame == 129), "identical_prefix": dsame}
         log(f"[bench] device session: prompt (127 tokens as one batch, the last as a step) {dp:.3f} s, 128 steps in {dd:.3f} s ({128 / dd:.0f} tok/s)")
         dev.close()
+        # Eight sequences decoded together (one token of each per step, the products as 8-token products): the
+        # continuous-batching shape.  Sequence 0 has the prompt above, so its tokens can be compared.
+        rngb = np.random.default_rng(seed + 1)
+        prompts = [prompt] + [rngb.integers(0, VOCAB, 128) for _ in range(7)]
+        bs = m.batch_session(8, 256, kv_block=16)
+        btoks, bp, bd = bs.generate_greedy(prompts, 64)
+        bsame = int(np.sum(np.cumprod(btoks[0] == dtoks[:64])))
+        out["batch_session"] = {"sequences": 8, "prompt_tokens": 8 * 128, "steps": 64, "prefill_s": round(bp, 3),
+                                "prefill_tok_per_s": round(8 * 127 / bp, 1), "decode_s": round(bd, 4),
+                                "decode_tok_per_s_all_sequences": round(8 * 64 / bd, 1), "ms_per_step": round(bd / 64 * 1e3, 3),
+                                "sequence_0_identical_prefix_to_single_session": bsame}
+        log(f"[bench] batch session: 8 sequences, 64 steps in {bd:.3f} s ({8 * 64 / bd:.0f} tok/s over all sequences)")
+        bs.close()
         m.close()
         if check_cpu:
             import oracle as O

@@ -76,6 +76,20 @@ int lnm_session_new(lnm_model *model, size_t kv_block, const uint32_t *block_ids
  * as a step; the environment variable LLAMA_HIP_DECODE_STEP_PREFILL makes every token a step. */
 int lnm_session_new_device(lnm_model *model, size_t kv_block, const uint32_t *block_ids, size_t n_block_ids,
                            size_t max_positions, lnm_session **out);
+/* A device session for `n_sequences` (at most 128) independent sequences of up to `max_positions` each, decoded
+ * together: every step processes one token of every sequence, the weight products as one multi-token product
+ * each (the continuous-batching shape of langtax/src/engine.rs:1423-1510, where M = the number of running
+ * sequences), attention per sequence over its own blocks of the paged cache.  Like the device session above it
+ * has no counterpart in the reference, whose batches return to the host after every product.  Freed with
+ * lnm_session_free; lnm_forward and lnm_generate_greedy refuse it. */
+int lnm_session_new_device_batch(lnm_model *model, size_t kv_block, size_t n_sequences, size_t max_positions,
+                                 lnm_session **out);
+/* Greedy decode of all sequences from scratch: `prompts` holds the prompts one after the other, prompt_lens[b]
+ * tokens for sequence b (at least 1); out[b * n_new + i] is token i of sequence b.  Prompts run one sequence
+ * after the other (all tokens but the last in chunks of up to 128, K and V only), then n_new steps of all
+ * sequences together, step 0 taking every prompt's last token. */
+int lnm_batch_generate_greedy(lnm_session *session, const uint32_t *prompts, const size_t *prompt_lens, size_t n_new,
+                              uint32_t *out, double *prefill_seconds, double *decode_seconds);
 void lnm_session_free(lnm_session *session);
 /* Runs the n tokens as one batch at positions past .. past+n-1 (products with n_tokens = n) and
  * writes the logits of the last one (n_vocab floats). */

@@ -131,6 +131,8 @@ def load_library():
         "lnm_set_products": (C.c_int, [vp, C.c_int, vp, vp]),
         "lnm_session_new": (C.c_int, [vp, sz, vp, sz, pvp]),
         "lnm_session_new_device": (C.c_int, [vp, sz, vp, sz, sz, pvp]),
+        "lnm_session_new_device_batch": (C.c_int, [vp, sz, sz, sz, pvp]),
+        "lnm_batch_generate_greedy": (C.c_int, [vp, vp, vp, sz, vp, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
         "lnm_session_free": (None, [vp]),
         "lnm_forward": (C.c_int, [vp, vp, sz, vp]),
         "lnm_generate_greedy": (C.c_int, [vp, vp, sz, sz, vp, C.POINTER(C.c_double), C.POINTER(C.c_double)]),

@@ -832,10 +832,31 @@ int lnm_session_new_device(lnm_model *model, size_t kv_block, const uint32_t *bl
     return 0;
 }
 
+int lnm_session_new_device_batch(lnm_model *model, size_t kv_block, size_t n_sequences, size_t max_positions,
+                                 lnm_session **out) {
+    lnm_session *s = nullptr;
+    if (lnm_session_new(model, kv_block, nullptr, 0, &s) != 0) return 1;
+    if (device_batch_create(s, n_sequences, max_positions) != 0) {
+        delete s;
+        *out = nullptr;
+        return 1;
+    }
+    *out = s;
+    return 0;
+}
+
+int lnm_batch_generate_greedy(lnm_session *session, const uint32_t *prompts, const size_t *prompt_lens, size_t n_new,
+                              uint32_t *out, double *prefill_seconds, double *decode_seconds) {
+    if (!session || !prompts || !prompt_lens || !out) return fail("null argument");
+    if (!session->dev || session->dev->n_seq == 0) return fail("not a batch session");
+    return device_batch_generate(session, prompts, prompt_lens, n_new, out, prefill_seconds, decode_seconds);
+}
+
 void lnm_session_free(lnm_session *session) { delete session; }
 
 int lnm_forward(lnm_session *session, const uint32_t *tokens, size_t n, float *logits) {
     if (!session || !tokens || !logits) return fail("null argument");
+    if (session->dev && session->dev->n_seq) return fail("a batch session takes lnm_batch_generate_greedy");
     if (session->dev) return device_forward(session, tokens, n, logits);
     return forward(session, tokens, n, logits);
 }
@@ -844,6 +865,7 @@ int lnm_generate_greedy(lnm_session *session, const uint32_t *prompt, size_t n_p
                         uint32_t *out, double *prefill_seconds, double *decode_seconds) {
     if (!session || !prompt || !out) return fail("null argument");
     if (n_prompt == 0 || n_new == 0) return fail("empty prompt or nothing to generate");
+    if (session->dev && session->dev->n_seq) return fail("a batch session takes lnm_batch_generate_greedy");
     if (session->dev) return device_generate(session, prompt, n_prompt, n_new, out, prefill_seconds, decode_seconds);
     std::vector<float> logits(session->model->hp.n_vocab);
     using clock = std::chrono::steady_clock;

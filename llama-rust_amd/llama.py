@@ -148,9 +148,43 @@ class Llama:
         """device_positions: keep the whole decode step on the GPU, with a cache of that many positions."""
         return Session(self, kv_block, block_ids, device_positions)
 
+    def batch_session(self, n_sequences, device_positions, kv_block=16):
+        """A device session that decodes `n_sequences` sequences together, one token of each per step."""
+        return BatchSession(self, n_sequences, device_positions, kv_block)
+
     def close(self):
         if self._h:
             _pkg.load_library().lnm_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class BatchSession:
+    def __init__(self, model, n_sequences, device_positions, kv_block=16):
+        self.model, self.n_sequences = model, n_sequences
+        h = C.c_void_p()
+        _check(_pkg.load_library().lnm_session_new_device_batch(model._h, kv_block, n_sequences, device_positions, C.byref(h)))
+        self._h = h
+
+    def generate_greedy(self, prompts, n_new):
+        """(tokens [n_sequences, n_new], prefill seconds, decode seconds) for one prompt per sequence."""
+        assert len(prompts) == self.n_sequences
+        flat = np.ascontiguousarray(np.concatenate([np.asarray(p, dtype=np.uint32) for p in prompts]), dtype=np.uint32)
+        lens = np.ascontiguousarray([len(p) for p in prompts], dtype=np.uintp)
+        out = np.empty((self.n_sequences, n_new), dtype=np.uint32)
+        tp, td = C.c_double(), C.c_double()
+        _check(_pkg.load_library().lnm_batch_generate_greedy(self._h, flat.ctypes.data, lens.ctypes.data, n_new,
+                                                             out.ctypes.data, C.byref(tp), C.byref(td)))
+        return out, tp.value, td.value
+
+    def close(self):
+        if self._h:
+            _pkg.load_library().lnm_session_free(self._h)
             self._h = None
 
     def __del__(self):

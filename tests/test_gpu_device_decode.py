@@ -217,6 +217,47 @@ def test_prompt_as_batches_equals_prompt_step_by_step(pkg, llama, tmp_path, monk
     assert ta.tolist() == tb.tolist()
 
 
+@pytest.mark.parametrize("n_seq,block_type", [(1, 12), (2, 12), (3, 2), (8, 12), (19, 8), (5, 14)])
+def test_batch_session_equals_independent_sessions(pkg, llama, tmp_path, n_seq, block_type):
+    """Sequences decoded together, one token of each per step (the weight products as one multi-token product:
+    single-token launches for 1 and 2 sequences, 16-token tiles up to 16, 32-token tiles above, and the 32-token
+    tiles for Q6_K), against every sequence decoded on its own in a device session: the same tokens.  Prompts
+    of different lengths, one of a single token, one longer than a prompt chunk."""
+    path = tmp_path / "small.gguf"
+    llama.write_synthetic_llama(path, n_layer=3, n_embd=512, n_head=8, n_head_kv=2, n_ff=1536, n_vocab=2048,
+                                block_type=block_type, seed=41)
+    m = llama.Llama(path=path)
+    rng = np.random.default_rng(100 + n_seq)
+    lens = [1, 150, 7, 33, 2, 64, 19, 5] + [int(v) for v in rng.integers(1, 40, 32)]
+    prompts = [rng.integers(0, 2048, lens[b]).tolist() for b in range(n_seq)]
+    n_new, cap = 14, 176
+    bs = m.batch_session(n_seq, cap)
+    together, _, _ = bs.generate_greedy(prompts, n_new)
+    for b in range(n_seq):
+        alone, _, _ = m.session(device_positions=cap).generate_greedy(prompts[b], n_new)
+        assert together[b].tolist() == alone.tolist(), f"sequence {b} of {n_seq}"
+    # a second generation in the same session starts every sequence afresh
+    again, _, _ = bs.generate_greedy(prompts[::-1], n_new)
+    assert again[::-1].tolist() == together.tolist()
+
+
+def test_batch_session_refuses_what_it_cannot_do(pkg, llama, tmp_path):
+    path = tmp_path / "small.gguf"
+    llama.write_synthetic_llama(path, n_layer=2, n_embd=256, n_head=4, n_head_kv=2, n_ff=512, n_vocab=512, seed=43)
+    m = llama.Llama(path=path)
+    with pytest.raises(Exception):
+        m.batch_session(129, 32)
+    s = m.batch_session(2, 32)
+    with pytest.raises(Exception):
+        s.generate_greedy([[1, 2, 3], [4] * 40], 4)  # 40 + 4 - 1 positions > 32
+    with pytest.raises(Exception):
+        s.generate_greedy([[1, 2, 3], []], 4)
+    with pytest.raises(Exception):
+        s.generate_greedy([[1, 2, 3], [600]], 4)  # token id out of range
+    out, _, _ = s.generate_greedy([[1, 2, 3], [4, 5]], 4)  # still usable
+    assert out.shape == (2, 4)
+
+
 @pytest.mark.parametrize("rows,cols,norm", [(14336, 4096, True), (14336, 4096, False), (1536, 2048, True), (1000, 8192, False)])
 def test_paired_swiglu_epilogue_equals_the_separate_steps(pkg, rows, cols, norm):
     """h = SiLU(gate x') * (up x') from one launch against float64 on the dequantized weights: each product
