@@ -563,8 +563,10 @@ int lnh_gemm_batch_device(lnh_exec *e, size_t n, const lnh_matrix *const *mats, 
             if (h == hipErrorInvalidValue) (void)hipGetLastError();
         }
         if (h == hipErrorInvalidValue) {
+            // consecutive multi-token products go out together: those of equal dtype and column count share launches
             run = 1;
-            int rc = launch_products(e, s, 1, &mats[i], &tokens[i], &dx[i], &dy[i]);
+            while (tokens[i] > 1 && i + run < n && tokens[i + run] > 1) run++;
+            int rc = launch_products(e, s, run, &mats[i], &tokens[i], &dx[i], &dy[i]);
             if (rc != LNH_OK) return rc;
             h = hipSuccess;
         }

@@ -476,6 +476,9 @@ static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *co
         job.y = ys ? ys[j] : nullptr;
         job.part = nullptr;
         job.tokens = tokens[j];
+        // products of the same activations (q, k, v of one input) read one set of split slots
+        const bool same_x = j > 0 && xs && xs[j] == xs[j - 1] && tokens[j] == tokens[j - 1];
+        if (same_x) total_tok -= tokens[j];
         job.tok_off = total_tok;
         job.wg_begin = wgs;
         job.tok_tiles = (tokens[j] + tile_tok - 1) / tile_tok;
