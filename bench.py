@@ -309,6 +309,13 @@ def greedy_decode(pkg, layers, check_cpu, seed):
                                 "sequence_0_identical_prefix_to_single_session": bsame}
         log(f"[bench] batch session: 8 sequences, 64 steps in {bd:.3f} s ({8 * 64 / bd:.0f} tok/s over all sequences)")
         bs.close()
+        prompts32 = prompts + [rngb.integers(0, VOCAB, 128) for _ in range(24)]
+        bs = m.batch_session(32, 192, kv_block=16)
+        _, bp32, bd32 = bs.generate_greedy(prompts32, 32)
+        out["batch_session_32"] = {"sequences": 32, "steps": 32, "prefill_tok_per_s": round(32 * 127 / bp32, 1),
+                                   "decode_tok_per_s_all_sequences": round(32 * 32 / bd32, 1), "ms_per_step": round(bd32 / 32 * 1e3, 3)}
+        log(f"[bench] batch session: 32 sequences, 32 steps in {bd32:.3f} s ({32 * 32 / bd32:.0f} tok/s over all sequences)")
+        bs.close()
         m.close()
         if check_cpu:
             import oracle as O
