@@ -128,7 +128,9 @@ int lnh_gemm_shared(lnh_exec *exec, size_t n_mats, const lnh_matrix *const *mats
  * Products of three or more tokens by a quantized matrix use a workspace that
  * belongs to the executor and grows on demand (growing allocates, so it cannot
  * happen while `stream` is being captured into a graph: run the largest shape
- * once before capturing).  Calls of one executor must therefore be enqueued on
+ * once before capturing; a workspace that captured launches point at stays
+ * allocated until the executor is destroyed, also after a later call has
+ * made the executor move to a larger one).  Calls of one executor must therefore be enqueued on
  * one stream at a time; calls that overlap on different streams race on it. */
 int lnh_gemm_device(lnh_exec *exec, const lnh_matrix *matrix, size_t tokens, const float *device_x,
                     float *device_y, void *stream);

@@ -43,6 +43,7 @@ struct lnh_exec {
     float *h_in = nullptr, *h_out = nullptr;  // pinned host staging for small calls, grow-only
     size_t hin_cap = 0, hout_cap = 0;
     void *d_ws = nullptr;                     // kernel workspace (multi-token products), grow-only
+    std::vector<void *> ws_retired;           // earlier, smaller workspaces: captured graphs may still point at them
     size_t ws_cap = 0;
     std::string err;
 };
@@ -134,21 +135,24 @@ bool ensure_pinned(lnh_exec *e, size_t in_floats, size_t out_floats) {
     return grow(e->h_in, e->hin_cap, in_floats) && grow(e->h_out, e->hout_cap, out_floats);
 }
 
-// Workspace of the multi-token kernels.  Work already queued that uses the old
-// buffer is safe: hipFree waits for the device before it releases memory.
+// Workspace of the multi-token kernels.  A workspace that has become too small is kept until the executor
+// goes: a caller may have captured launches that point at it into a HIP graph (a decode step that is replayed
+// while another call, a longer prompt say, makes the workspace grow), and work already queued may still use
+// it.  Growth is by at least half, so everything retired together is smaller than twice the live buffer.
 int ensure_workspace(lnh_exec *e, size_t bytes) {
     if (bytes <= e->ws_cap) return LNH_OK;
-    if (e->d_ws) (void)hipFree(e->d_ws);
-    e->d_ws = nullptr;
-    e->ws_cap = 0;
-    size_t want = bytes + bytes / 4;
-    hipError_t h = hipMalloc(&e->d_ws, want);
+    size_t want = bytes > e->ws_cap + e->ws_cap / 2 ? bytes : e->ws_cap + e->ws_cap / 2;
+    want += want / 4;
+    void *fresh = nullptr;
+    hipError_t h = hipMalloc(&fresh, want);
     if (h != hipSuccess) {
         (void)hipGetLastError();
         want = bytes;
-        h = hipMalloc(&e->d_ws, want);
+        h = hipMalloc(&fresh, want);
     }
     if (h != hipSuccess) return hip_fail(e, h, "HIP workspace allocation");
+    if (e->d_ws) e->ws_retired.push_back(e->d_ws);
+    e->d_ws = fresh;
     e->ws_cap = want;
     return LNH_OK;
 }
@@ -355,6 +359,7 @@ void lnh_destroy(lnh_exec *e) {
         (void)hipStreamDestroy(e->stream);
     }
     if (e->d_ws) (void)hipFree(e->d_ws);
+    for (void *p : e->ws_retired) (void)hipFree(p);
     if (e->d_in) (void)hipFree(e->d_in);
     if (e->d_out) (void)hipFree(e->d_out);
     if (e->h_in) (void)hipHostFree(e->h_in);

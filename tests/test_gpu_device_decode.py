@@ -236,7 +236,10 @@ def test_batch_session_equals_independent_sessions(pkg, llama, tmp_path, n_seq, 
     for b in range(n_seq):
         alone, _, _ = m.session(device_positions=cap).generate_greedy(prompts[b], n_new)
         assert together[b].tolist() == alone.tolist(), f"sequence {b} of {n_seq}"
-    # a second generation in the same session starts every sequence afresh
+    # A second generation in the same session starts every sequence afresh.  In between the executor's workspace
+    # has grown (128-token prompt chunks above, a 300-token host batch here): the session's captured step still
+    # points at the workspace it was captured with, which therefore must not have been freed.
+    m.session().forward(rng.integers(0, 2048, 300).tolist())
     again, _, _ = bs.generate_greedy(prompts[::-1], n_new)
     assert again[::-1].tolist() == together.tolist()
 
