@@ -542,6 +542,16 @@ static hipError_t launch_mm16_main(hipStream_t stream, const MmBatch &b) {
     return hipGetLastError();
 }
 
+// Workgroups per job of the share reduction: one float4 per thread where that fills fewer than 512.
+static uint32_t mm_reduce_blocks(const MmBatch &b) {
+    size_t most = 1;
+    for (uint32_t j = 0; j < b.n_jobs; j++) {
+        const size_t vec = ((size_t)b.job[j].tokens * b.job[j].m.rows + 3) / 4, blocks = (vec + 255) / 256;
+        if (b.job[j].ksplit > 1 && blocks > most) most = blocks;
+    }
+    return (uint32_t)(most < 512 ? most : 512);
+}
+
 template <uint32_t T>
 static hipError_t launch_mm_t(hipStream_t stream, MmPlan &p, void *ws, size_t ws_bytes) {
     if (p.xb_bytes + p.sx_bytes + p.part_bytes > ws_bytes) return hipErrorInvalidValue;
@@ -562,7 +572,7 @@ static hipError_t launch_mm_t(hipStream_t stream, MmPlan &p, void *ws, size_t ws
         if (p.tile16) {
             e = launch_mm16_main<T>(stream, b);
             if (e != hipSuccess) return e;
-            if (b.any_split) hipLaunchKernelGGL(mm_reduce_kernel, dim3(512, b.n_jobs), dim3(256), 0, stream, b);
+            if (b.any_split) hipLaunchKernelGGL(mm_reduce_kernel, dim3(mm_reduce_blocks(b), b.n_jobs), dim3(256), 0, stream, b);
             return hipGetLastError();
         }
     }
@@ -572,7 +582,7 @@ static hipError_t launch_mm_t(hipStream_t stream, MmPlan &p, void *ws, size_t ws
     else if (p.max_tok <= 24) e = launch_mm_main<T, 1, 3>(stream, b);
     else e = launch_mm_main<T, 1, 4>(stream, b);
     if (e != hipSuccess) return e;
-    if (b.any_split) hipLaunchKernelGGL(mm_reduce_kernel, dim3(512, b.n_jobs), dim3(256), 0, stream, b);
+    if (b.any_split) hipLaunchKernelGGL(mm_reduce_kernel, dim3(mm_reduce_blocks(b), b.n_jobs), dim3(256), 0, stream, b);
     return hipGetLastError();
 }
 
