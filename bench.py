@@ -488,6 +488,10 @@ def main():
             # step resident on the GPU, and through the reference's host seam (one round trip per product)
             out["decode_tok_per_s_end_to_end"] = e2e["device_session"]["decode_tok_per_s"]
             out["decode_tok_per_s_host_seam"] = e2e["decode_tok_per_s"]
+            # the same model with 8 and 32 sequences decoded together (not batch 1: beside the metric, not in it)
+            out["decode_tok_per_s_8_sequences"] = e2e["batch_session"]["decode_tok_per_s_all_sequences"]
+            out["decode_tok_per_s_32_sequences"] = e2e["batch_session_32"]["decode_tok_per_s_all_sequences"]
+            out["prompt_tok_per_s_device_session"] = e2e["device_session"]["prefill_tok_per_s"]
             out["greedy_tokens_identical_to_cpu_path"] = bool(e2e.get("tokens_identical")) and bool(
                 e2e["device_session"].get("tokens_identical_to_cpu_path")) if args.e2e_check else None
     if args.cpu_seconds > 0:
