@@ -136,6 +136,19 @@ int lnh_gemm_device(lnh_exec *exec, const lnh_matrix *matrix, size_t tokens, con
                     float *device_y, void *stream);
 int lnh_gemm_grouped_device(lnh_exec *exec, size_t n_groups, const lnh_matrix *const *mats,
                             const size_t *tokens, const float *device_x, float *device_y, void *stream);
+/* lnh_gemm_device for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid it).  No counterpart in the reference.  Same product, same
+ * kernels, same results as lnh_gemm_device, but the workspace of the multi-token kernels is a fixed
+ * array inside the library's device code (LNH_NOALLOC_WORKSPACE_BYTES per GPU, held from lnh_create on
+ * that GPU until the process ends) instead of the executor's grow-on-demand allocation: the call
+ * never allocates or frees.  A product that needs more fails with LNH_ERR_INVALID
+ * (the message states the need) before anything is launched.  Every call on one GPU, from any executor, uses the
+ * same array and nothing in it outlives a call: calls that may overlap on one GPU (different streams,
+ * different threads) race on it and must be ordered by the caller. */
+#define LNH_NOALLOC_WORKSPACE_BYTES ((size_t)64 << 20)
+int lnh_gemm_device_noalloc(lnh_exec *exec, const lnh_matrix *matrix, size_t tokens, const float *device_x,
+                            float *device_y, void *stream);
+
 /* n independent products enqueued back to back in one call: product i multiplies
  * tokens[i] rows at device_x[i] by mats[i] into device_y[i].  This is how a decode
  * step's products (langtax/src/decode.rs:2755-2996: q, k, v, o, gate, up, down per

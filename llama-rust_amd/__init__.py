@@ -104,6 +104,7 @@ def load_library():
         "lnh_gemm_shared": (C.c_int, [vp, sz, pvp, sz, vp, sz, vp, sz]),
         "lnh_gemm_device": (C.c_int, [vp, vp, sz, vp, vp, vp]),
         "lnh_gemm_grouped_device": (C.c_int, [vp, sz, pvp, psz, vp, vp, vp]),
+        "lnh_gemm_device_noalloc": (C.c_int, [vp, vp, sz, vp, vp, vp]),
         "lnh_gemm_batch_device": (C.c_int, [vp, sz, pvp, psz, pvp, pvp, vp]),
         "lnh_gemv_shared_device": (C.c_int, [vp, sz, pvp, vp, pvp, C.c_int, vp]),
         "lnh_gemv_fused_device": (C.c_int, [vp, sz, pvp, vp, pvp, C.c_int, C.c_int, vp, C.c_float, vp]),
@@ -313,6 +314,11 @@ class HipGemv:
     def gemm_device(self, matrix, tokens, x_ptr, y_ptr, stream=0):
         self._check(self._lib.lnh_gemm_device(self._h, matrix._h, tokens, C.c_void_p(x_ptr), C.c_void_p(y_ptr),
                                               C.c_void_p(stream)))
+
+    def gemm_device_noalloc(self, matrix, tokens, x_ptr, y_ptr, stream=0):
+        """gemm_device with the library's fixed device workspace: never allocates (include/native_hip.h)."""
+        self._check(self._lib.lnh_gemm_device_noalloc(self._h, matrix._h, tokens, C.c_void_p(x_ptr), C.c_void_p(y_ptr),
+                                                      C.c_void_p(stream)))
 
     def gemm_grouped_device(self, matrices, tokens, x_ptr, y_ptr, stream=0):
         n = len(matrices)

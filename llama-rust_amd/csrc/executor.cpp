@@ -15,6 +15,8 @@
 #include "../../include/native_hip.h"
 #include "kernels.h"
 
+static_assert(LNH_NOALLOC_WORKSPACE_BYTES == nh::STATIC_SCRATCH_BYTES, "header and device array disagree");
+
 namespace {
 
 struct Ctx {
@@ -347,6 +349,13 @@ int lnh_create(int device_ordinal, lnh_exec **out) {
         return hip_fail(nullptr, h, "fp8 unpack probe");
     }
     nh::set_fp8_nibble_unit(unit);
+    // address of this device's copy of the static workspace (lnh_gemm_device_noalloc), looked up while
+    // the device is current
+    h = nh::static_scratch_init(device_ordinal);
+    if (h != hipSuccess) {
+        (void)hipStreamDestroy(e->stream);
+        return hip_fail(nullptr, h, "hipGetSymbolAddress(static workspace)");
+    }
     *out = e.release();
     return LNH_OK;
 }
@@ -517,6 +526,25 @@ int lnh_gemm_device(lnh_exec *e, const lnh_matrix *m, size_t tokens, const float
     if (!dx || !dy) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
     hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
     return launch_products(e, s, 1, &m, &tokens, &dx, &dy);
+}
+
+int lnh_gemm_device_noalloc(lnh_exec *e, const lnh_matrix *m, size_t tokens, const float *dx, float *dy, void *stream) {
+    size_t inputs, outputs;
+    int rc = check_gemm(e, m, tokens, false, 0, 0, &inputs, &outputs);
+    if (rc != LNH_OK) return rc;
+    if (!dx || !dy) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    void *ws = nh::static_scratch(e->ctx->device);
+    if (!ws) return fail(e, LNH_ERR_DEVICE, "static workspace of this device was not initialised");
+    const uint32_t tok32 = (uint32_t)tokens;
+    const size_t need = nh::gemm_workspace_bytes(&m->view, &tok32, 1);
+    if (need > nh::STATIC_SCRATCH_BYTES)
+        return fail(e, LNH_ERR_INVALID,
+                    "product needs " + std::to_string(need) + " bytes of workspace, the allocation-free entry point holds " +
+                        std::to_string(nh::STATIC_SCRATCH_BYTES) + ": use lnh_gemm_device or fewer tokens per call");
+    hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
+    const hipError_t h = nh::launch_gemm_groups(s, &m->view, &m->tiled, &tok32, &dx, &dy, 1, ws, nh::STATIC_SCRATCH_BYTES);
+    if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
+    return LNH_OK;
 }
 
 int lnh_gemm_grouped_device(lnh_exec *e, size_t n_groups, const lnh_matrix *const *mats, const size_t *tokens,

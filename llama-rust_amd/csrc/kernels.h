@@ -53,6 +53,15 @@ hipError_t launch_gemv_multi_prologue(hipStream_t stream, const MatView *mats, f
 hipError_t launch_gemv_swiglu_pair(hipStream_t stream, const MatView &gate, const MatView &up, const float *x, float *h,
                                    int prologue, const float *x2, float eps);
 
+// Device memory that belongs to the code object instead of an allocation: STATIC_SCRATCH_BYTES per GPU,
+// usable as the workspace of launch_gemm_groups by callers that may not allocate.
+// static_scratch_init(device) looks the address up (the device must be current; once per device,
+// repeated calls are free); static_scratch(device) returns it, null before that.  Everything that
+// uses it on one GPU shares it: such launches must not overlap.
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)64 << 20;
+hipError_t static_scratch_init(int device);
+void *static_scratch(int device);
+
 // dst[0, nbytes) = src[0, nbytes) (nbytes a multiple of 16): reference traffic for counter calibration.
 hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t nbytes);
 // The same copy with a grid sized by nbytes: activations between pinned host staging memory (which the

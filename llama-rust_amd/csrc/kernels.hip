@@ -726,6 +726,33 @@ hipError_t launch_copy_small(hipStream_t stream, void *dst, const void *src, siz
     return hipGetLastError();
 }
 
+// ---- device memory that no call allocates
+//
+// Workspace of the multi-token kernels (split activations, their group sums, partial results of
+// column shares) for callers that may not allocate: a file-scope device array, one copy per GPU that
+// loads this code object, held until the process ends.  In host code the array's name only stands for
+// the symbol; its device address comes from hipGetSymbolAddress, once per device, and only that
+// address is ever handed to kernels.
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+constexpr int SCRATCH_MAX_DEVICES = 64;
+static void *g_scratch_ptr[SCRATCH_MAX_DEVICES];  // per device ordinal, null until static_scratch_init
+
+hipError_t static_scratch_init(int device) {
+    if (device < 0 || device >= SCRATCH_MAX_DEVICES) return hipErrorInvalidDevice;
+    if (g_scratch_ptr[device]) return hipSuccess;
+    void *ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));  // of the current device
+    if (e != hipSuccess) return e;
+    if (!ptr) return hipErrorInvalidSymbol;
+    g_scratch_ptr[device] = ptr;
+    return hipSuccess;
+}
+
+void *static_scratch(int device) {
+    return device >= 0 && device < SCRATCH_MAX_DEVICES ? g_scratch_ptr[device] : nullptr;
+}
+
 hipError_t launch_gemv_multi(hipStream_t stream, const MatView *mats, float *const *ys, uint32_t n, const float *x,
                              bool accumulate) {
     if (n == 0) return hipSuccess;
