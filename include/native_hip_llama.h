@@ -1,5 +1,5 @@
 /*
- * native-hip, host side of a dense Llama decode: the caller of the matrix products.
+ * native-hip, host side of a Llama decode (dense or routed feed-forward): the caller of the matrix products.
  *
  * The matrix executor (native_hip.h) replaces one seam of the reference; this header is
  * the code either side of that seam, restated in C++ so that an end-to-end greedy decode
@@ -7,7 +7,7 @@
  *
  *   GGUF v3 reader / writer             langtax/src/gguf.rs:64-68, 626-702, 728-828, 922-947
  *   model load (llama architecture)     langtax/src/decode.rs:1910-1958, 2050-2090, 7461-7475
- *   forward pass of n tokens            langtax/src/decode.rs:2710-3099 (dense llama branch)
+ *   forward pass of n tokens            langtax/src/decode.rs:2710-3099 (llama branch; routed experts 9938-10292)
  *     RMSNorm 11498-11513, RoPE (adjacent pairs) 11578-11602, attention 11126-11197,
  *     softmax 12021-12033, SiLU 11826-11830, argmax 12104-12114, embedding 10761-10800
  *   paged K/V addressing                langtax/src/kv_page.rs:410-438, decode.rs:12059-12100
@@ -40,6 +40,7 @@ typedef struct lnm_hparams {
     uint32_t n_layer, n_embd, n_head, n_head_kv, n_ff, n_vocab, head_dim, n_rot;
     float rope_base, rms_eps;
     uint32_t block_type, embd_type, output_type; /* ggml type ids of blk.0.attn_q, token_embd, output */
+    uint32_t n_expert, n_expert_used;            /* llama.expert_count / expert_used_count; 0, 0: dense feed-forward */
 } lnm_hparams;
 
 enum { LNM_PRODUCTS_RESIDENT = 0, LNM_PRODUCTS_DISPATCH = 1, LNM_PRODUCTS_CALLBACK = 2 };
@@ -111,6 +112,15 @@ int lnm_rmsnorm(float *x, const float *w, size_t n, float eps);
 int lnm_rope(float *head, size_t head_len, size_t pos, size_t n_rot, float base);
 void lnm_softmax(float *x, size_t n);
 uint32_t lnm_argmax(const float *x, size_t n);
+/* Routed feed-forward (langtax/src/decode.rs:9938-10116, 10148-10292, 10366-10409).
+ * lnm_topk: indices of the k largest of n values, descending, ties to the lower index (decode.rs:11363-11379).
+ * lnm_router_weights: weights[j] = probs[order[j]], divided by max(their sum, 2^-14) when norm_w (decode.rs:11391-11409).
+ * lnm_moe_ffn: the whole routed feed-forward of `layer` on n_tokens rows x (n_embd each, already normed) by the
+ * model's product route: router product, softmax, top-k, renormalised weights, tokens bucketed per expert in
+ * ascending expert order, gate / up products, SiLU(gate) * up, down product, ffn_out[t] += y * w. */
+int lnm_topk(const float *values, size_t n, size_t k, uint32_t *order);
+int lnm_router_weights(const float *probs, const uint32_t *order, size_t k, int norm_w, float *weights);
+int lnm_moe_ffn(lnm_model *model, size_t layer, size_t n_tokens, const float *x, float *ffn_out);
 
 /* A random dense llama model written as GGUF v3: packed blocks are drawn directly (codes uniform,
  * block scales sized so that the dequantized weights have mean 0 and standard deviation
@@ -120,6 +130,7 @@ typedef struct lnm_synth_spec {
     uint32_t block_type, embd_type, output_type; /* ggml type ids */
     float rope_base, rms_eps, weight_std;
     uint64_t seed;
+    uint32_t n_expert, n_expert_used; /* > 0: routed feed-forward (ffn_gate_inp F32 + 3-D ffn_{gate,up,down}_exps of block_type) */
 } lnm_synth_spec;
 int lnm_write_synthetic_llama(const char *gguf_path, const lnm_synth_spec *spec);
 

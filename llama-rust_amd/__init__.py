@@ -139,6 +139,9 @@ def load_library():
         "lnm_generate_greedy": (C.c_int, [vp, vp, sz, sz, vp, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
         "lnm_session_timing": (C.c_int, [vp, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_uint64)]),
         "lnm_dequant_row": (C.c_int, [u32, sz, vp, sz, vp]),
+        "lnm_topk": (C.c_int, [vp, sz, sz, vp]),
+        "lnm_router_weights": (C.c_int, [vp, vp, sz, C.c_int, vp]),
+        "lnm_moe_ffn": (C.c_int, [vp, sz, sz, vp, vp]),
         "lnm_rmsnorm": (C.c_int, [vp, vp, sz, C.c_float]),
         "lnm_rope": (C.c_int, [vp, sz, sz, sz, C.c_float]),
         "lnm_softmax": (None, [vp, sz]),

@@ -96,13 +96,19 @@ bool read_value(Reader &r, int32_t ty, Kv *out, int depth, std::string *err) {
     case KV_ARRAY: {
         out->elem = r.get<int32_t>();
         const uint64_t n = r.get<uint64_t>();
-        if (!r.ok || depth > 4 || n > r.n) {  // every element takes at least one byte
+        // every element takes at least one byte of what is left; the vector grows with the elements
+        // actually read, so a huge count in a short file cannot reserve memory up front
+        if (!r.ok || depth > 4 || n > r.n - r.pos) {
             *err = "truncated";
             return false;
         }
-        out->items.resize((size_t)n);
-        for (auto &it : out->items)
+        out->items.clear();
+        out->items.reserve((size_t)(n < 4096 ? n : 4096));
+        for (uint64_t i = 0; i < n; i++) {
+            Kv it;
             if (!read_value(r, out->elem, &it, depth + 1, err)) return false;
+            out->items.push_back(std::move(it));
+        }
         break;
     }
     default: *err = "unsupported metadata type " + std::to_string(ty); return false;
@@ -180,8 +186,11 @@ bool parse(const uint8_t *bytes, size_t size, File *out, std::string *err) {
             if (d != 0 && n_el > UINT64_MAX / d) return *err = "bad shape", false;
             n_el *= d;
         }
-        if (n_el % k != 0) return *err = "bad shape", false;
-        const uint64_t nbytes = n_el / k * block;
+        // rows are whole blocks (the row dequantizers and the device kernels walk a row block by block)
+        if (t.shape[0] % k != 0) return *err = "bad shape", false;
+        const uint64_t n_blocks = n_el / k;
+        if (n_blocks > UINT64_MAX / block) return *err = "bad shape", false;
+        const uint64_t nbytes = n_blocks * block;
         if (t.offset > size || data_start > size - (size_t)t.offset) return *err = "truncated", false;
         const size_t start = data_start + (size_t)t.offset;
         if (nbytes > size - start) return *err = "truncated", false;

@@ -11,6 +11,7 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <cmath>
@@ -216,6 +217,38 @@ uint32_t argmax(const float *x, size_t n) {  // first maximum wins; langtax/src/
     return (uint32_t)best_i;
 }
 
+// Indices of the k largest values, descending, ties to the lower index (langtax/src/decode.rs:11363-11379:
+// ggml_argsort_top_k; a NaN compares as a tie).  False when k is 0 or exceeds n.
+bool topk(const float *v, size_t n, size_t k, std::vector<uint32_t> *order) {
+    if (k == 0 || k > n) return false;
+    order->resize(n);
+    for (size_t i = 0; i < n; i++) (*order)[i] = (uint32_t)i;
+    std::sort(order->begin(), order->end(), [&](uint32_t a, uint32_t b) {
+        const float va = v[a], vb = v[b];
+        if (vb < va) return true;    // a first: larger value
+        if (vb > va) return false;
+        return a < b;                // equal or unordered: lower index first
+    });
+    order->resize(k);
+    return true;
+}
+
+// Official build_moe_ffn norm_w clamp: the smallest normal f16 (decode.rs:321).
+constexpr float MOE_NORM_W_CLAMP = 1.0f / 16384.0f;
+
+// Router weights of the selected experts (decode.rs:11391-11409): their probabilities, renormalised to sum
+// one when norm_w, with the sum clamped from below.
+void router_weights(const float *probs, const uint32_t *order, size_t k, bool norm_w, float *w) {
+    float wsum = 0.f;
+    for (size_t j = 0; j < k; j++) {
+        w[j] = probs[order[j]];
+        wsum += w[j];
+    }
+    if (!norm_w) return;
+    if (wsum < MOE_NORM_W_CLAMP) wsum = MOE_NORM_W_CLAMP;
+    for (size_t j = 0; j < k; j++) w[j] /= wsum;
+}
+
 // ------------------------------------------------------------------ worker threads for the attention heads
 
 // The reference attends head after head on one thread.  Heads are independent, so they are
@@ -296,6 +329,19 @@ struct Mat {
 struct Layer {
     std::vector<float> attn_norm, ffn_norm;
     Mat wq, wk, wv, wo, gate, up, down;
+    // Routed feed-forward (llama.expert_count > 0, langtax/src/decode.rs:569-577, 9228-9256): the router and
+    // the experts' gate / up / down matrices, expert e being part e of the 3-D *_exps tensors
+    // (decode.rs:9853-9913: bytes [start + e * per, start + (e + 1) * per)).
+    bool moe = false;
+    Mat gate_inp;
+    std::vector<Mat> gate_e, up_e, down_e;
+};
+
+// Scratch of the routed feed-forward (langtax/src/decode.rs:1530-1560, MoeScratch).
+struct MoeScratch {
+    std::vector<float> logits, sel_w, pack_x, g, u, y;
+    std::vector<uint32_t> sel_e, order;
+    std::vector<std::vector<uint32_t>> buckets;
 };
 
 }  // namespace
@@ -319,8 +365,11 @@ struct lnm_model {
             if (m.resident) lnh_matrix_free(m.resident);
             m.resident = nullptr;
         };
-        for (Layer &l : layers)
-            for (Mat *m : {&l.wq, &l.wk, &l.wv, &l.wo, &l.gate, &l.up, &l.down}) drop(*m);
+        for (Layer &l : layers) {
+            for (Mat *m : {&l.wq, &l.wk, &l.wv, &l.wo, &l.gate, &l.up, &l.down, &l.gate_inp}) drop(*m);
+            for (auto *v : {&l.gate_e, &l.up_e, &l.down_e})
+                for (Mat &m : *v) drop(m);
+        }
         drop(token_embd);
         drop(output);
         if (exec) lnh_destroy(exec);
@@ -340,6 +389,7 @@ struct lnm_session {
     // q, k, v share one buffer (matrix after matrix), and so do gate and up: products of one
     // input can then be fetched by a single call
     std::vector<float> x, residual, qkv, attn, attn_proj, gate_up, ffn_out, xn;
+    MoeScratch moe;
     double products_s = 0.0, attention_s = 0.0;  // wall time spent in weight products / in attend + RoPE
     uint64_t n_products = 0;
     std::unique_ptr<HeadPool> pool;
@@ -368,6 +418,30 @@ bool read_mat(const nh::gguf::File &f, const std::string &name, size_t n_rows, s
     out->n_cols = n_cols;
     out->bytes = f.data + t->start;
     out->nbytes = t->end - t->start;
+    return true;
+}
+
+// A 3-D tensor [n_cols, n_rows, n_parts] (ggml order) as n_parts matrices over consecutive byte ranges
+// (langtax/src/decode.rs:476-493, 9853-9913).  n_rows or n_cols given as 0 is taken from the tensor.
+bool read_parts(const nh::gguf::File &f, const std::string &name, size_t n_parts, size_t n_rows, size_t n_cols,
+                std::vector<Mat> *out, std::string *err) {
+    const nh::gguf::TensorInfo *t = f.tensor(name);
+    if (!t) return *err = "missing tensor " + name, false;
+    if (t->shape.size() != 3 || t->shape[2] != n_parts || (n_cols && t->shape[0] != n_cols) ||
+        (n_rows && t->shape[1] != n_rows))
+        return *err = "tensor " + name + " has the wrong shape", false;
+    const size_t total = t->end - t->start, per = total / n_parts;
+    if (per * n_parts != total) return *err = "tensor " + name + " does not split into its parts", false;
+    out->resize(n_parts);
+    for (size_t e = 0; e < n_parts; e++) {
+        Mat &m = (*out)[e];
+        m.name = name + "[" + std::to_string(e) + "]";
+        m.type = t->type;
+        m.n_rows = (size_t)t->shape[1];
+        m.n_cols = (size_t)t->shape[0];
+        m.bytes = f.data + t->start + e * per;
+        m.nbytes = per;
+    }
     return true;
 }
 
@@ -407,6 +481,14 @@ int finish_load(lnm_model *m) {
     } else {
         m->output = m->token_embd;  // tied head (decode.rs:2069-2072)
     }
+    // decode.rs:8502-8519: a missing or zero llama.expert_count is a dense model
+    hp.n_expert = hp.n_expert_used = 0;
+    uint32_t n_expert = 0;
+    if (f.kv_u32(arch + ".expert_count", &n_expert) && n_expert != 0) {
+        if (!need_u32("expert_used_count", &hp.n_expert_used)) return fail(err);
+        if (hp.n_expert_used == 0 || hp.n_expert_used > n_expert) return fail("bad " + arch + ".expert_used_count");
+        hp.n_expert = n_expert;
+    }
     const size_t qw = (size_t)hp.n_head * hp.head_dim, kvw = (size_t)hp.n_head_kv * hp.head_dim;
     m->layers.resize(hp.n_layer);
     for (uint32_t i = 0; i < hp.n_layer; i++) {
@@ -417,11 +499,25 @@ int finish_load(lnm_model *m) {
             !read_mat(f, p + "attn_q.weight", qw, hp.n_embd, &l.wq, &err) ||
             !read_mat(f, p + "attn_k.weight", kvw, hp.n_embd, &l.wk, &err) ||
             !read_mat(f, p + "attn_v.weight", kvw, hp.n_embd, &l.wv, &err) ||
-            !read_mat(f, p + "attn_output.weight", hp.n_embd, qw, &l.wo, &err) ||
-            !read_mat(f, p + "ffn_gate.weight", hp.n_ff, hp.n_embd, &l.gate, &err) ||
-            !read_mat(f, p + "ffn_up.weight", hp.n_ff, hp.n_embd, &l.up, &err) ||
-            !read_mat(f, p + "ffn_down.weight", hp.n_embd, hp.n_ff, &l.down, &err))
+            !read_mat(f, p + "attn_output.weight", hp.n_embd, qw, &l.wo, &err))
             return fail(err);
+        if (hp.n_expert == 0) {
+            if (!read_mat(f, p + "ffn_gate.weight", hp.n_ff, hp.n_embd, &l.gate, &err) ||
+                !read_mat(f, p + "ffn_up.weight", hp.n_ff, hp.n_embd, &l.up, &err) ||
+                !read_mat(f, p + "ffn_down.weight", hp.n_embd, hp.n_ff, &l.down, &err))
+                return fail(err);
+            continue;
+        }
+        // decode.rs:9228-9256: the router has one row per expert, the three expert tensors one part per expert,
+        // gate and up agree on the hidden width and down takes it back to n_embd
+        l.moe = true;
+        if (!read_mat(f, p + "ffn_gate_inp.weight", hp.n_expert, hp.n_embd, &l.gate_inp, &err)) return fail(err);
+        if (!read_parts(f, p + "ffn_gate_exps.weight", hp.n_expert, 0, hp.n_embd, &l.gate_e, &err) ||
+            !read_parts(f, p + "ffn_up_exps.weight", hp.n_expert, 0, hp.n_embd, &l.up_e, &err) ||
+            !read_parts(f, p + "ffn_down_exps.weight", hp.n_expert, hp.n_embd, 0, &l.down_e, &err))
+            return fail(err);
+        if (l.gate_e[0].n_rows != l.up_e[0].n_rows || l.down_e[0].n_cols != l.up_e[0].n_rows)
+            return fail("blk." + std::to_string(i) + ".ffn_*_exps.weight disagree on the hidden width");
     }
     hp.block_type = m->layers[0].wq.type;
     hp.embd_type = m->token_embd.type;
@@ -525,7 +621,126 @@ int ensure_blocks(lnm_session *s, size_t positions) {
     return 0;
 }
 
-// langtax/src/decode.rs:2710-3099, dense llama branch, LogitsKind::Last.
+// Uploads w once (RESIDENT route).
+int ensure_resident(lnm_model *m, Mat &w) {
+    if (!m->exec && lnh_create(0, &m->exec) != 0) return fail(std::string("executor: ") + lnh_thread_error());
+    if (!w.resident && lnh_upload_packed(m->exec, w.type, w.n_rows, w.n_cols, w.bytes, w.nbytes, &w.resident) != 0)
+        return fail(std::string(lnh_last_error(m->exec)) + " (" + w.name + ")");
+    return 0;
+}
+
+// One projection of every non-empty expert: expert e multiplies its counts[e] packed rows.  The reference
+// issues one product per expert (decode.rs:10035-10058, 10148-10261: gemm_part_bytes_into, which takes the
+// single-token route for one row); the RESIDENT route hands all of them to the executor in one grouped call.
+int expert_products(lnm_model *m, std::vector<Mat> &parts, const std::vector<size_t> &counts, const float *x, float *y,
+                    lnm_session *timed) {
+    const auto t0 = wall_clock::now();
+    size_t n_calls = 0;
+    if (m->route == LNM_PRODUCTS_RESIDENT) {
+        std::vector<const lnh_matrix *> handles;
+        std::vector<size_t> toks;
+        size_t x_len = 0, y_len = 0;
+        for (size_t e = 0; e < parts.size(); e++) {
+            if (counts[e] == 0) continue;
+            if (ensure_resident(m, parts[e]) != 0) return 1;
+            handles.push_back(parts[e].resident);
+            toks.push_back(counts[e]);
+            x_len += counts[e] * parts[e].n_cols;
+            y_len += counts[e] * parts[e].n_rows;
+        }
+        if (!handles.empty() &&
+            lnh_gemm_grouped(m->exec, handles.size(), handles.data(), toks.data(), x, x_len, y, y_len) != 0)
+            return fail(std::string(lnh_last_error(m->exec)) + " (" + parts[0].name + ")");
+        n_calls = handles.size();
+    } else {
+        for (size_t e = 0; e < parts.size(); e++) {
+            if (counts[e] == 0) continue;
+            if (product_routed(m, parts[e], counts[e], x, y) != 0) return 1;
+            x += counts[e] * parts[e].n_cols;
+            y += counts[e] * parts[e].n_rows;
+            n_calls++;
+        }
+    }
+    if (timed) {
+        timed->products_s += since(t0);
+        timed->n_products += n_calls;
+    }
+    return 0;
+}
+
+// The routed feed-forward of architecture llama with experts (Mixtral-shaped), langtax/src/decode.rs:10366-10409
+// (llama_moe_into: softmax over all experts, then top-k, weights renormalised with the 2^-14 clamp and applied
+// after the expert, SwiGLU, no shared expert), through softmax_routed_layer 9938-9966:
+//   route_softmax_tokens 9969-10004   router product, per token softmax -> topk -> router weights
+//   grouped_routed_ffn 10006-10060    token indices bucketed per expert, experts in ascending order
+//   grouped_one_expert 10062-10116    the bucket's rows packed contiguously
+//   swiglu_expert_gemm 10148-10261    gate and up products, SiLU(gate) * up, down product
+//   scatter_expert_rows 10263-10292   ffn_out[t] += y[i] * w(t, e)
+// x: n x n_embd rows (already normed), ffn_out: n x n_embd, overwritten.
+int moe_ffn(lnm_model *m, Layer &l, size_t n, const float *x, float *ffn_out, MoeScratch *ms, lnm_session *timed) {
+    const lnm_hparams &hp = m->hp;
+    const size_t d = hp.n_embd, ne = hp.n_expert, k = hp.n_expert_used, ff = l.gate_e[0].n_rows;
+    ms->logits.resize(n * ne);
+    {
+        const auto t0 = wall_clock::now();
+        if (product_routed(m, l.gate_inp, n, x, ms->logits.data()) != 0) return 1;
+        if (timed) {
+            timed->products_s += since(t0);
+            timed->n_products++;
+        }
+    }
+    ms->sel_e.resize(n * k);
+    ms->sel_w.resize(n * k);
+    for (size_t t = 0; t < n; t++) {
+        float *row = &ms->logits[t * ne];
+        softmax(row, ne);
+        if (!topk(row, ne, k, &ms->order)) return fail("expert_used_count");
+        std::copy(ms->order.begin(), ms->order.end(), &ms->sel_e[t * k]);
+        router_weights(row, ms->order.data(), k, true, &ms->sel_w[t * k]);
+    }
+    ms->buckets.resize(ne);
+    for (auto &b : ms->buckets) b.clear();
+    for (size_t t = 0; t < n; t++)
+        for (size_t j = 0; j < k; j++) ms->buckets[ms->sel_e[t * k + j]].push_back((uint32_t)t);
+    std::vector<size_t> counts(ne);
+    size_t pairs = 0;
+    for (size_t e = 0; e < ne; e++) pairs += counts[e] = ms->buckets[e].size();
+    // every expert's rows, expert after expert in ascending order
+    ms->pack_x.resize(pairs * d);
+    ms->g.resize(pairs * ff);
+    ms->u.resize(pairs * ff);
+    ms->y.resize(pairs * d);
+    size_t at = 0;
+    for (size_t e = 0; e < ne; e++)
+        for (uint32_t t : ms->buckets[e]) std::memcpy(&ms->pack_x[at++ * d], x + (size_t)t * d, d * sizeof(float));
+    if (expert_products(m, l.gate_e, counts, ms->pack_x.data(), ms->g.data(), timed)) return 1;
+    if (expert_products(m, l.up_e, counts, ms->pack_x.data(), ms->u.data(), timed)) return 1;
+    for (size_t i = 0; i < pairs * ff; i++) {  // silu_inplace then the element-wise product, decode.rs:10244-10248
+        const float g = ms->g[i];
+        ms->g[i] = g / (1.f + std::exp(-g));
+        ms->g[i] *= ms->u[i];
+    }
+    if (expert_products(m, l.down_e, counts, ms->g.data(), ms->y.data(), timed)) return 1;
+    std::fill(ffn_out, ffn_out + n * d, 0.f);  // fit() zero-fills (decode.rs:1816-1819, 10381)
+    at = 0;
+    for (size_t e = 0; e < ne; e++) {
+        for (uint32_t t : ms->buckets[e]) {
+            float w = 0.f;  // token_expert_weight: the first selection of this expert by the token
+            for (size_t j = 0; j < k; j++)
+                if (ms->sel_e[(size_t)t * k + j] == e) {
+                    w = ms->sel_w[(size_t)t * k + j];
+                    break;
+                }
+            const float *src = &ms->y[at++ * d];
+            float *dst = ffn_out + (size_t)t * d;
+            const float scale = 1.f;  // no ffn_down_exps.scale tensor on this architecture (expert_part_scale)
+            for (size_t i = 0; i < d; i++) dst[i] += src[i] * w * scale;
+        }
+    }
+    return 0;
+}
+
+// langtax/src/decode.rs:2710-3099, llama branch (dense or routed feed-forward), LogitsKind::Last.
 int forward(lnm_session *s, const uint32_t *tokens, size_t n, float *logits) {
     lnm_model *m = s->model;
     const lnm_hparams &hp = m->hp;
@@ -601,13 +816,17 @@ int forward(lnm_session *s, const uint32_t *tokens, size_t n, float *logits) {
         for (size_t i = 0; i < n * d; i++) s->x[i] = s->attn_proj[i] + s->residual[i];
         s->residual = s->x;
         for (size_t t = 0; t < n; t++) rmsnorm(&s->x[t * d], l.ffn_norm.data(), d, hp.rms_eps);
-        if (products_shared(s, {&l.gate, &l.up}, n, s->x.data(), gate)) return 1;
-        for (size_t i = 0; i < n * hp.n_ff; i++) {  // SiLU(gate) * up, decode.rs:11826-11830 and 2981-2984
-            const float g = gate[i];
-            gate[i] = g / (1.f + std::exp(-g));
-            gate[i] *= up[i];
+        if (l.moe) {
+            if (moe_ffn(m, l, n, s->x.data(), s->ffn_out.data(), &s->moe, s)) return 1;
+        } else {
+            if (products_shared(s, {&l.gate, &l.up}, n, s->x.data(), gate)) return 1;
+            for (size_t i = 0; i < n * hp.n_ff; i++) {  // SiLU(gate) * up, decode.rs:11826-11830 and 2981-2984
+                const float g = gate[i];
+                gate[i] = g / (1.f + std::exp(-g));
+                gate[i] *= up[i];
+            }
+            if (product(s, l.down, n, gate, s->ffn_out.data())) return 1;
         }
-        if (product(s, l.down, n, gate, s->ffn_out.data())) return 1;
         for (size_t i = 0; i < n * d; i++) s->x[i] = s->ffn_out[i] + s->residual[i];
     }
     s->xn.assign(s->x.begin() + (n - 1) * d, s->x.begin() + n * d);
@@ -752,10 +971,14 @@ const char *lnm_last_error(void) { return t_err.c_str(); }
 int lnm_load_bytes(const uint8_t *bytes, size_t len, lnm_model **out) {
     if (!bytes || !out) return fail("null argument");
     std::unique_ptr<lnm_model> m(new lnm_model);
-    m->owned.assign(bytes, bytes + len);
-    std::string err;
-    if (!nh::gguf::parse(m->owned.data(), m->owned.size(), &m->file, &err)) return fail("gguf: " + err);
-    if (finish_load(m.get()) != 0) return 1;
+    try {
+        m->owned.assign(bytes, bytes + len);
+        std::string err;
+        if (!nh::gguf::parse(m->owned.data(), m->owned.size(), &m->file, &err)) return fail("gguf: " + err);
+        if (finish_load(m.get()) != 0) return 1;
+    } catch (const std::exception &e) {  // allocation failure on a hostile file must not cross the C boundary
+        return fail(std::string("gguf: ") + e.what());
+    }
     *out = m.release();
     return 0;
 }
@@ -775,9 +998,13 @@ int lnm_load(const char *path, lnm_model **out) {
     std::unique_ptr<lnm_model> m(new lnm_model);
     m->map = p;
     m->map_len = (size_t)st.st_size;
-    std::string err;
-    if (!nh::gguf::parse(static_cast<const uint8_t *>(p), m->map_len, &m->file, &err)) return fail("gguf: " + err);
-    if (finish_load(m.get()) != 0) return 1;
+    try {
+        std::string err;
+        if (!nh::gguf::parse(static_cast<const uint8_t *>(p), m->map_len, &m->file, &err)) return fail("gguf: " + err);
+        if (finish_load(m.get()) != 0) return 1;
+    } catch (const std::exception &e) {
+        return fail(std::string("gguf: ") + e.what());
+    }
     *out = m.release();
     return 0;
 }
@@ -918,6 +1145,32 @@ void lnm_softmax(float *x, size_t n) {
 
 uint32_t lnm_argmax(const float *x, size_t n) { return x ? argmax(x, n) : 0; }
 
+int lnm_topk(const float *values, size_t n, size_t k, uint32_t *order) {
+    if (!values || !order) return fail("null argument");
+    std::vector<uint32_t> o;
+    if (!topk(values, n, k, &o)) return fail("expert_used_count");
+    std::copy(o.begin(), o.end(), order);
+    return 0;
+}
+
+int lnm_router_weights(const float *probs, const uint32_t *order, size_t k, int norm_w, float *weights) {
+    if (!probs || !order || !weights) return fail("null argument");
+    router_weights(probs, order, k, norm_w != 0, weights);
+    return 0;
+}
+
+int lnm_moe_ffn(lnm_model *model, size_t layer, size_t n_tokens, const float *x, float *ffn_out) {
+    if (!model || !x || !ffn_out) return fail("null argument");
+    if (layer >= model->layers.size() || !model->layers[layer].moe) return fail("layer has no routed feed-forward");
+    if (n_tokens == 0) return fail("empty batch");
+    try {
+        MoeScratch ms;
+        return moe_ffn(model, model->layers[layer], n_tokens, x, ffn_out, &ms, nullptr);
+    } catch (const std::exception &e) {
+        return fail(std::string("routed feed-forward: ") + e.what());
+    }
+}
+
 int lnm_write_synthetic_llama(const char *path, const lnm_synth_spec *sp) {
     if (!path || !sp) return fail("null argument");
     if (!sp->n_layer || !sp->n_embd || !sp->n_head || !sp->n_head_kv || !sp->n_ff || !sp->n_vocab)
@@ -945,21 +1198,30 @@ int lnm_write_synthetic_llama(const char *path, const lnm_synth_spec *sp) {
         {"llama.attention.layer_norm_rms_epsilon", Kv::f32(sp->rms_eps)},
         {"llama.vocab_size", Kv::u32(sp->n_vocab)},
     };
+    if (sp->n_expert) {
+        if (sp->n_expert_used == 0 || sp->n_expert_used > sp->n_expert) return fail("bad expert_used_count");
+        kv.push_back({"llama.expert_count", Kv::u32(sp->n_expert)});
+        kv.push_back({"llama.expert_used_count", Kv::u32(sp->n_expert_used)});
+    }
     std::vector<nh::gguf::TensorWrite> tensors;
     uint64_t serial = 0;
     const uint64_t seed = sp->seed;
     const float sigma = sp->weight_std;
-    auto mat = [&](const std::string &name, uint32_t type, size_t n_rows, size_t n_cols) {
+    // n_parts > 1: a 3-D tensor [n_cols, n_rows, n_parts], part after part; sd: deviation of the weights
+    auto mat = [&](const std::string &name, uint32_t type, size_t n_rows, size_t n_cols, size_t n_parts = 1, float sd = -1.f) {
         nh::gguf::TensorWrite t;
         t.name = name;
         t.type = type;
         t.shape = {n_cols, n_rows};
+        if (n_parts > 1) t.shape.push_back(n_parts);
         size_t b = 0, k = 0;
         nh::gguf::type_layout(type, &b, &k);
-        t.nbytes = n_rows * (n_cols / k * b);
+        const size_t all_rows = n_rows * n_parts;
+        t.nbytes = all_rows * (n_cols / k * b);
         uint64_t st = seed + 0x9e3779b97f4a7c15ull * ++serial;
         const uint64_t tensor_seed = splitmix(st);
-        t.fill = [=](uint8_t *dst) { random_rows(type, n_cols, n_rows, sigma, tensor_seed, dst); };
+        const float dev = sd < 0.f ? sigma : sd;
+        t.fill = [=](uint8_t *dst) { random_rows(type, n_cols, all_rows, dev, tensor_seed, dst); };
         tensors.push_back(std::move(t));
     };
     auto norm = [&](const std::string &name) {
@@ -988,9 +1250,17 @@ int lnm_write_synthetic_llama(const char *path, const lnm_synth_spec *sp) {
         mat(p + "attn_v.weight", sp->block_type, kvw, d);
         mat(p + "attn_output.weight", sp->block_type, d, qw);
         norm(p + "ffn_norm.weight");
-        mat(p + "ffn_gate.weight", sp->block_type, sp->n_ff, d);
-        mat(p + "ffn_up.weight", sp->block_type, sp->n_ff, d);
-        mat(p + "ffn_down.weight", sp->block_type, d, sp->n_ff);
+        if (sp->n_expert) {
+            // router rows of deviation 1 / sqrt(n_embd): logits of about unit deviation on normed activations
+            mat(p + "ffn_gate_inp.weight", 0, sp->n_expert, d, 1, 1.0f / std::sqrt((float)d));
+            mat(p + "ffn_gate_exps.weight", sp->block_type, sp->n_ff, d, sp->n_expert);
+            mat(p + "ffn_up_exps.weight", sp->block_type, sp->n_ff, d, sp->n_expert);
+            mat(p + "ffn_down_exps.weight", sp->block_type, d, sp->n_ff, sp->n_expert);
+        } else {
+            mat(p + "ffn_gate.weight", sp->block_type, sp->n_ff, d);
+            mat(p + "ffn_up.weight", sp->block_type, sp->n_ff, d);
+            mat(p + "ffn_down.weight", sp->block_type, d, sp->n_ff);
+        }
     }
     norm("output_norm.weight");
     mat("output.weight", sp->output_type, sp->n_vocab, d);

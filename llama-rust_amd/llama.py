@@ -24,13 +24,14 @@ class HParams(C.Structure):
     _fields_ = [(n, C.c_uint32) for n in ("n_layer", "n_embd", "n_head", "n_head_kv", "n_ff", "n_vocab",
                                             "head_dim", "n_rot")] + \
                [("rope_base", C.c_float), ("rms_eps", C.c_float)] + \
-               [(n, C.c_uint32) for n in ("block_type", "embd_type", "output_type")]
+               [(n, C.c_uint32) for n in ("block_type", "embd_type", "output_type", "n_expert", "n_expert_used")]
 
 
 class SynthSpec(C.Structure):
     _fields_ = [(n, C.c_uint32) for n in ("n_layer", "n_embd", "n_head", "n_head_kv", "n_ff", "n_vocab",
                                             "block_type", "embd_type", "output_type")] + \
-               [("rope_base", C.c_float), ("rms_eps", C.c_float), ("weight_std", C.c_float), ("seed", C.c_uint64)]
+               [("rope_base", C.c_float), ("rms_eps", C.c_float), ("weight_std", C.c_float), ("seed", C.c_uint64),
+                ("n_expert", C.c_uint32), ("n_expert_used", C.c_uint32)]
 
 
 class LlamaError(RuntimeError):
@@ -44,9 +45,10 @@ def _check(rc):
 
 def write_synthetic_llama(path, *, n_layer, n_embd, n_head, n_head_kv, n_ff, n_vocab, block_type=_pkg.Q4_K,
                           embd_type=_pkg.Q4_K, output_type=_pkg.Q6_K, rope_base=5e5, rms_eps=1e-5,
-                          weight_std=0.02, seed=0):
+                          weight_std=0.02, seed=0, n_expert=0, n_expert_used=0):
+    """n_expert > 0: every layer's feed-forward is routed over that many experts, n_expert_used per token."""
     spec = SynthSpec(n_layer, n_embd, n_head, n_head_kv, n_ff, n_vocab, block_type, embd_type, output_type,
-                     rope_base, rms_eps, weight_std, seed)
+                     rope_base, rms_eps, weight_std, seed, n_expert, n_expert_used)
     _check(_pkg.load_library().lnm_write_synthetic_llama(str(path).encode(), C.byref(spec)))
 
 
@@ -106,6 +108,22 @@ def argmax(x):
     return _pkg.load_library().lnm_argmax(v.ctypes.data, v.size)
 
 
+def topk(values, k):
+    """Indices of the k largest values, descending, ties to the lower index."""
+    v = np.ascontiguousarray(values, dtype=np.float32)
+    order = np.empty(k, dtype=np.uint32)
+    _check(_pkg.load_library().lnm_topk(v.ctypes.data, v.size, k, order.ctypes.data))
+    return order
+
+
+def router_weights(probs, order, norm_w=True):
+    p = np.ascontiguousarray(probs, dtype=np.float32)
+    o = np.ascontiguousarray(order, dtype=np.uint32)
+    w = np.empty(o.size, dtype=np.float32)
+    _check(_pkg.load_library().lnm_router_weights(p.ctypes.data, o.ctypes.data, o.size, int(norm_w), w.ctypes.data))
+    return w
+
+
 class Llama:
     """A loaded model; `products` picks the route of the weight products."""
 
@@ -143,6 +161,13 @@ class Llama:
             cb = MATMUL_FN(thunk)
         _check(lib.lnm_set_products(self._h, route, C.cast(cb, C.c_void_p) if cb else None, None))
         self._cb = cb  # keep the thunk alive
+
+    def moe_ffn(self, layer, x):
+        """The routed feed-forward of `layer` on the rows x [n_tokens, n_embd] (already normed)."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        out = np.empty_like(x)
+        _check(_pkg.load_library().lnm_moe_ffn(self._h, layer, x.shape[0], x.ctypes.data, out.ctypes.data))
+        return out
 
     def session(self, kv_block=16, block_ids=None, device_positions=None):
         """device_positions: keep the whole decode step on the GPU, with a cache of that many positions."""

@@ -105,3 +105,50 @@ def test_8b_layer_shapes_generate_the_same_tokens_as_the_simd_cpu_path(pkg, llam
     toks_g, toks_c, worst, margins = run_both(llama, path, prompt, 16, simd=True, threads=0)
     assert toks_g == toks_c, (toks_g, toks_c, min(margins))
     assert worst <= 1e-4, worst
+
+
+# ------------------------------------------------------------------ routed experts (llama with expert_count > 0)
+
+@pytest.mark.parametrize("block_type", [12, 2])
+def test_small_model_with_experts_generates_the_same_tokens_as_the_cpu_path(pkg, llama, tmp_path, block_type):
+    """A 4-expert top-2 model (langtax/tests/native_cuda_parity.rs:198-288 runs its MoE tiny the same way):
+    the host routing is shared, the router and expert products run on the GPU - as one grouped call per
+    projection (resident route) and as one call per expert through the content-identified dispatch layer,
+    the reference's call shape - against the CPU oracle's products."""
+    path = tmp_path / "moe.gguf"
+    llama.write_synthetic_llama(path, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, n_ff=768, n_vocab=1024,
+                                block_type=block_type, embd_type=block_type, output_type=8, seed=21,
+                                weight_std=0.06, n_expert=4, n_expert_used=2)
+    rng = np.random.default_rng(4)
+    prompt = rng.integers(0, 1024, 21).tolist()
+    toks_g, toks_c, worst, margins = run_both(llama, path, prompt, 20, simd=False, threads=1)
+    assert toks_g == toks_c, (toks_g, toks_c, min(margins))
+    assert worst <= 1e-4, worst
+    pkg.load_library().lnq_reset()
+    toks_d, _, worst_d, _ = run_both(llama, path, prompt, 20, simd=False, threads=1, products=llama.DISPATCH)
+    assert toks_d == toks_c
+    assert worst_d <= 1e-4, worst_d
+    assert len(set(toks_c)) >= 15  # the layers matter: no fixed point, no short cycle
+
+
+def test_mixtral_shaped_routed_layer_matches_the_cpu_path(pkg, llama, tmp_path):
+    """Benchmark configuration 5 as one checked result: 64 tokens, router logits of about unit deviation,
+    softmax, top-2 of 8 experts, tokens grouped per expert, Q4_K gate / up (4096 -> 14336) and down
+    (14336 -> 4096), weighted scatter-add - the whole layer on the GPU route against the same host code over
+    the AVX2 restatement of the reference's CPU kernels.  Tolerance: every output within 1e-4 of
+    max(|e|, rms(e) / 4), the relative criterion of the product tests applied to the layer's output."""
+    path = tmp_path / "mixtral_layer.gguf"
+    llama.write_synthetic_llama(path, n_layer=1, n_embd=4096, n_head=32, n_head_kv=8, n_ff=14336, n_vocab=256,
+                                block_type=12, embd_type=8, output_type=8, seed=8, n_expert=8, n_expert_used=2)
+    gpu = llama.Llama(path=path)
+    cpu = llama.Llama(path=path, products=llama.CALLBACK, matmul=cpu_products(True, 0))
+    rng = np.random.default_rng(64)
+    x = rng.normal(0, 1, (64, 4096)).astype(np.float32)
+    got, want = gpu.moe_ffn(0, x), cpu.moe_ffn(0, x)
+    rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    assert rms > 0 and np.all(np.isfinite(got))
+    err = np.abs(got.astype(np.float64) - want)
+    assert np.all(err <= 1e-4 * np.maximum(np.abs(want), rms / 4)), float((err / np.maximum(np.abs(want), rms / 4)).max())
+    # one token alone takes the single-token kernels for its two experts: same row up to summation order
+    alone = gpu.moe_ffn(0, x[5:6])
+    assert np.all(np.abs(alone[0].astype(np.float64) - want[5]) <= 1e-4 * np.maximum(np.abs(want[5]), rms / 4))

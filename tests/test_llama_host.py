@@ -203,56 +203,7 @@ def test_softmax_and_argmax(llama):
 
 # ------------------------------------------------------------------ forward pass
 
-def numpy_forward(blob, tensors, hp, tokens, n_past_kv=None):
-    """Independent float64 restatement of the dense llama forward over dequantized weights: logits of
-    every position (causal attention, adjacent-pair RoPE, GQA, SwiGLU)."""
-    by = {t[0]: t for t in tensors}
-
-    def mat(name):
-        _, ty, shape, start, end = by[name]
-        n_cols, n_rows = shape
-        return oracle.dequant(ty, n_cols, blob[start:end], n_rows).astype(np.float64)
-
-    def vec(name):
-        _, _, _, start, end = by[name]
-        return blob[start:end].view(np.float32).astype(np.float64)
-
-    d, hd, n_head, n_kv = hp.n_embd, hp.head_dim, hp.n_head, hp.n_head_kv
-    eps, base, n_rot = float(hp.rms_eps), float(hp.rope_base), hp.n_rot
-    n = len(tokens)
-
-    def norm(x, w):
-        return x / np.sqrt((x ** 2).mean(axis=-1, keepdims=True) + eps) * w
-
-    def rot(v):  # v: [n, heads, hd]
-        i = np.arange(n_rot // 2)
-        th = np.arange(n)[:, None] * base ** (-2.0 * i / n_rot)[None, :]
-        z = (v[..., 0:n_rot:2] + 1j * v[..., 1:n_rot:2]) * np.exp(1j * th)[:, None, :]
-        out = v.copy()
-        out[..., 0:n_rot:2], out[..., 1:n_rot:2] = z.real, z.imag
-        return out
-
-    x = mat("token_embd.weight")[np.asarray(tokens)]
-    for li in range(hp.n_layer):
-        p = f"blk.{li}."
-        h = norm(x, vec(p + "attn_norm.weight"))
-        q = rot((h @ mat(p + "attn_q.weight").T).reshape(n, n_head, hd))
-        k = rot((h @ mat(p + "attn_k.weight").T).reshape(n, n_kv, hd))
-        v = (h @ mat(p + "attn_v.weight").T).reshape(n, n_kv, hd)
-        att = np.zeros((n, n_head, hd))
-        for hq in range(n_head):
-            kk, vv = k[:, hq // (n_head // n_kv)], v[:, hq // (n_head // n_kv)]
-            sc = q[:, hq] @ kk.T / np.sqrt(hd)
-            sc[np.triu_indices(n, 1)] = -np.inf
-            pr = np.exp(sc - sc.max(axis=1, keepdims=True))
-            pr /= pr.sum(axis=1, keepdims=True)
-            att[:, hq] = pr @ vv
-        x = x + att.reshape(n, -1) @ mat(p + "attn_output.weight").T
-        h = norm(x, vec(p + "ffn_norm.weight"))
-        g = h @ mat(p + "ffn_gate.weight").T
-        u = h @ mat(p + "ffn_up.weight").T
-        x = x + (g / (1 + np.exp(-g)) * u) @ mat(p + "ffn_down.weight").T
-    return norm(x, vec("output_norm.weight")) @ mat("output.weight").T
+from llama_ref import numpy_forward  # noqa: E402  (independent float64 forward, shared with the routed-expert tests)
 
 
 def test_model_load_reads_the_hyper_parameters(llama, pkg, tiny_path):
