@@ -250,9 +250,12 @@ int check_packed_shape(lnh_exec *e, uint32_t type, size_t rows, size_t cols, siz
     if (cols > UINT32_MAX) return fail(e, LNH_ERR_INVALID, "GEMV columns exceed u32");
     size_t rb = nh::gguf_row_bytes(type, cols), total;
     if (rb == 0 || mul_overflows(rb, rows, &total)) return fail(e, LNH_ERR_INVALID, "GEMV shape overflow");
-    if (nbytes != total) return fail(e, LNH_ERR_INVALID, "GEMV buffer lengths do not match shape");
     // plane strides are kept in 32 bits
     if (nh::plane_spec(type, 1, cols).stride[0] > UINT32_MAX) return fail(e, LNH_ERR_INVALID, "GEMV columns exceed u32");
+    // the Q4_K single-token kernel forms byte offsets inside a plane in 32 bits
+    if (type == nh::T_Q4_K && rows * nh::plane_spec(type, 1, cols).stride[0] > UINT32_MAX)
+        return fail(e, LNH_ERR_INVALID, "Q4_K matrix exceeds 4 GiB of codes: split it by rows");
+    if (nbytes != total) return fail(e, LNH_ERR_INVALID, "GEMV buffer lengths do not match shape");
     return LNH_OK;
 }
 

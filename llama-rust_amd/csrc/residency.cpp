@@ -149,10 +149,25 @@ int ensure_state() {
     return LNH_OK;
 }
 
+// A freshly uploaded matrix that enters the cache once the product that needed it has succeeded
+// (native_gpu.rs:190-211 pushes the entry after gemm_resident returns Ok): a failed product leaves no
+// charged entry behind.
+struct Pending {
+    bool keep = false;
+    Entry entry;
+};
+
+void commit(State &s, Pending &p) {
+    if (!p.keep) return;
+    s.bytes += p.entry.bytes;
+    s.cache.push_back(std::move(p.entry));
+    p.keep = false;
+}
+
 // Resident matrix for these bytes: hit -> move to back, miss -> evict from the
-// front until it fits, upload packed, keep if within budget.
+// front until it fits, upload packed; `pending` then holds the entry to keep if within budget.
 int resident(State &s, uint32_t type, size_t rows, size_t cols, const uint8_t *w, size_t w_len,
-             std::shared_ptr<Holder> *out) {
+             std::shared_ptr<Holder> *out, Pending *pending) {
     WeightKey key = make_key(type, rows, cols, w, w_len);
     for (size_t i = 0; i < s.cache.size(); i++) {
         Entry &en = s.cache[i];
@@ -178,13 +193,11 @@ int resident(State &s, uint32_t type, size_t rows, size_t cols, const uint8_t *w
     if (rc != LNH_OK) return qfail(rc, lnh_last_error(s.gpu));
     *out = holder;
     if (bytes <= s.limit) {
-        s.bytes += bytes;
-        Entry en;
-        en.key = key;
-        en.packed.assign(w, w + w_len);
-        en.matrix = holder;
-        en.bytes = bytes;
-        s.cache.push_back(std::move(en));
+        pending->keep = true;
+        pending->entry.key = key;
+        pending->entry.packed.assign(w, w + w_len);
+        pending->entry.matrix = holder;
+        pending->entry.bytes = bytes;
     }
     return LNH_OK;
 }
@@ -219,16 +232,19 @@ int lnq_gemm(uint32_t type, size_t n_cols, size_t n_tokens, const uint8_t *w, si
     int rc = check_matmul(type, n_cols, n_tokens, w_len, x_len, y_len, &n_rows);
     if (rc != LNH_OK) return rc;
     if (n_rows == 0) return LNH_OK;
+    if (!w || !x || !y) return qfail(LNH_ERR_INVALID, "buffer pointer is null");
     if (t_state && t_state->busy) return qfail(LNH_ERR_INVALID, "recursive GPU execution is unsupported");
     rc = ensure_state();
     if (rc != LNH_OK) return rc;
     State &s = *t_state;
     BusyGuard guard(&s);
     std::shared_ptr<Holder> mat;
-    rc = resident(s, type, n_rows, n_cols, w, w_len, &mat);
+    Pending pending;
+    rc = resident(s, type, n_rows, n_cols, w, w_len, &mat, &pending);
     if (rc != LNH_OK) return rc;
     rc = lnh_gemm(s.gpu, mat->m, n_tokens, x, x_len, y, y_len);
     if (rc != LNH_OK) return qfail(rc, lnh_last_error(s.gpu));
+    commit(s, pending);
     return LNH_OK;
 }
 
@@ -258,12 +274,16 @@ int lnq_gemm_grouped(uint32_t type, size_t n_cols, size_t n_rows, size_t n_group
     if (x_len != total * n_cols) return size_error("X F32 elems", x_len, total * n_cols);
     if (y_len != total * n_rows) return size_error("Y F32 elems", y_len, total * n_rows);
     if (total == 0) return LNH_OK;
+    if (!x || !y) return qfail(LNH_ERR_INVALID, "buffer pointer is null");
+    for (size_t g = 0; g < n_groups; g++)
+        if (tokens[g] != 0 && !parts[g]) return qfail(LNH_ERR_INVALID, "buffer pointer is null");
     if (t_state && t_state->busy) return qfail(LNH_ERR_INVALID, "recursive GPU execution is unsupported");
     int rc = ensure_state();
     if (rc != LNH_OK) return rc;
     State &s = *t_state;
     BusyGuard guard(&s);
     std::vector<std::shared_ptr<Holder>> holders(n_groups);
+    std::vector<Pending> pending(n_groups);
     std::vector<const lnh_matrix *> mats(n_groups, nullptr);
     std::vector<size_t> toks(tokens, tokens + n_groups);
     // Experts without tokens are skipped before their weights are touched
@@ -271,7 +291,9 @@ int lnq_gemm_grouped(uint32_t type, size_t n_cols, size_t n_rows, size_t n_group
     const lnh_matrix *any = nullptr;
     for (size_t g = 0; g < n_groups; g++) {
         if (toks[g] == 0) continue;
-        rc = resident(s, type, n_rows, n_cols, parts[g], part_len, &holders[g]);
+        // parts uploaded earlier in this call are not in the cache yet: a part that repeats is uploaded again,
+        // which costs time, never correctness
+        rc = resident(s, type, n_rows, n_cols, parts[g], part_len, &holders[g], &pending[g]);
         if (rc != LNH_OK) return rc;
         mats[g] = holders[g]->m;
         any = mats[g];
@@ -280,6 +302,17 @@ int lnq_gemm_grouped(uint32_t type, size_t n_cols, size_t n_rows, size_t n_group
         if (!mats[g]) mats[g] = any;  // placeholder for skipped groups (tokens == 0)
     rc = lnh_gemm_grouped(s.gpu, n_groups, mats.data(), toks.data(), x, x_len, y, y_len);
     if (rc != LNH_OK) return qfail(rc, lnh_last_error(s.gpu));
+    for (size_t g = 0; g < n_groups; g++) {
+        // the budget may have been consumed by the parts committed before this one
+        if (pending[g].keep && admission_requires_eviction(s.bytes, pending[g].entry.bytes, s.limit)) {
+            while (!s.cache.empty() && admission_requires_eviction(s.bytes, pending[g].entry.bytes, s.limit)) {
+                s.bytes = s.bytes > s.cache.front().bytes ? s.bytes - s.cache.front().bytes : 0;
+                s.cache.pop_front();
+            }
+            if (admission_requires_eviction(s.bytes, pending[g].entry.bytes, s.limit)) pending[g].keep = false;
+        }
+        commit(s, pending[g]);
+    }
     return LNH_OK;
 }
 

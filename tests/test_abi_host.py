@@ -127,6 +127,15 @@ def test_invalid_matrix_operations_preserve_output_without_touching_the_device(p
     assert pkg.load_library().lnq_gemm(pkg.F32, USIZE_MAX, 2, None, 0, None, 0, out.ctypes.data, 1) != 0
     assert pkg.load_library().lnq_gemm(pkg.F32, USIZE_MAX, 2, None, 0, None, 0, out.ctypes.data, 0) != 0
     assert out[0] == np.float32(123.5)
+    # lengths that are right with a pointer that is not: refused before the device is touched
+    x32, y1 = np.zeros(32, np.float32), np.array([123.5], np.float32)
+    lib = pkg.load_library()
+    assert lib.lnq_gemm(pkg.Q8_0, 32, 1, None, 34, x32.ctypes.data, 32, y1.ctypes.data, 1) != 0
+    assert b"buffer pointer is null" in lib.lnq_last_error()
+    w34 = np.zeros(34, np.uint8)
+    assert lib.lnq_gemm(pkg.Q8_0, 32, 1, w34.ctypes.data, 34, None, 32, y1.ctypes.data, 1) != 0
+    assert lib.lnq_gemm(pkg.Q8_0, 32, 1, w34.ctypes.data, 34, x32.ctypes.data, 32, None, 1) != 0
+    assert y1[0] == np.float32(123.5)
     with pytest.raises(pkg.NativeHipError, match="n_cols 33 is not a multiple of 32"):
         pkg.gemv(pkg.Q8_0, 33, np.zeros(34, np.uint8), np.zeros(33, np.float32), np.zeros(1, np.float32))
     with pytest.raises(pkg.NativeHipError, match="unsupported GGUF dtype"):

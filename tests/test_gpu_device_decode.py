@@ -48,6 +48,25 @@ def test_device_session_matches_the_host_session(pkg, llama, tmp_path, block_typ
     assert td.tolist() == th.tolist()
 
 
+@pytest.mark.parametrize("head_dim", [192, 256])
+def test_device_session_with_large_heads(pkg, llama, tmp_path, head_dim):
+    """Head sizes beyond 128 need more than 48 KB of LDS in both attention kernels (the single step and the
+    prompt batch): the step and a 40-token prompt give the host session's tokens."""
+    path = tmp_path / "wide_heads.gguf"
+    llama.write_synthetic_llama(path, n_layer=2, n_embd=2 * head_dim, n_head=2, n_head_kv=1, n_ff=1024, n_vocab=512,
+                                block_type=8, embd_type=8, output_type=8, seed=31, weight_std=0.06)
+    m = llama.Llama(path=path)
+    assert m.hparams.head_dim == head_dim
+    rng = np.random.default_rng(7)
+    prompt = rng.integers(0, 512, 40).tolist()
+    th, _, _ = m.session().generate_greedy(prompt, 10)
+    td, _, _ = m.session(device_positions=64).generate_greedy(prompt, 10)
+    assert td.tolist() == th.tolist()
+    # a block table too long for the device's LDS is refused with the figures, before anything is launched
+    with pytest.raises(llama.LlamaError, match="bytes of LDS"):
+        m.session(kv_block=1, device_positions=1 << 16)
+
+
 def test_device_session_pages_and_capacity(pkg, llama, tmp_path):
     """Any physical block order and block size gives the same tokens; running past the cache is an error
     raised before anything is launched."""

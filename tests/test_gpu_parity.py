@@ -231,6 +231,40 @@ def test_invalid_operations_preserve_output_with_a_live_device(pkg):
         assert again[0] == ok[0]
 
 
+def test_q4k_matrix_beyond_32_bit_plane_offsets_is_refused(pkg, gpu):
+    """The Q4_K single-token kernel addresses a plane with 32-bit byte offsets: an upload whose code plane
+    would reach 4 GiB is refused by shape, before any byte of it is read (the buffer here is a stub)."""
+    stub = np.zeros(144, np.uint8)
+    with pytest.raises(pkg.NativeHipError, match="exceeds 4 GiB of codes") as ei:
+        gpu.upload_packed(K.Q4_K, 65536, 131072, stub)
+    assert ei.value.code == pkg.ERR_INVALID
+    m = gpu.upload_packed(K.Q4_K, 1, 256, stub)  # the executor is still usable
+    m.close()
+
+
+def test_a_failed_product_leaves_no_cache_entry_behind(pkg):
+    """langtax/src/native_gpu.rs:190-211 keeps an uploaded matrix only after its product returned Ok."""
+    pkg.reset()
+    rng = np.random.default_rng(12)
+    cols, rows = 64, 5
+    w = K.random_packed(K.Q8_0, rows, cols, rng)
+    x = rng.normal(0, 1, cols).astype(np.float32)
+    y = np.zeros(rows, np.float32)
+    pkg.gemv(K.Q8_0, cols, w, x, y)
+    before = pkg.cache_stats()
+    assert before["entries"] == 1 and before["misses"] == 1
+    # tokens * rows beyond u32: passes native_matmul's checks, is uploaded, and the product is refused
+    lib = pkg.load_library()
+    w2 = K.random_packed(K.Q8_0, 1, 32, rng)
+    huge = (1 << 32) + 8
+    rc = lib.lnq_gemm(K.Q8_0, 32, huge, w2.ctypes.data, w2.size, x.ctypes.data, huge * 32, y.ctypes.data, huge)
+    assert rc != 0 and b"exceeds u32" in lib.lnq_last_error()
+    after = pkg.cache_stats()
+    assert after["entries"] == 1 and after["bytes"] == before["bytes"] and after["misses"] == 2
+    pkg.gemv(K.Q8_0, cols, w, x, y)  # the earlier entry is still there and still found
+    assert pkg.cache_stats()["hits"] == before["hits"] + 1
+
+
 # ------------------------------------------------------------------ random data, all dtypes
 @pytest.mark.parametrize("ty", O.ALL_TYPES, ids=lambda t: O.TYPE_NAMES[t])
 def test_random_gemv_and_gemm_within_bounds(pkg, gpu, ty):

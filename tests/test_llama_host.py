@@ -118,6 +118,43 @@ def test_handwritten_gguf_with_every_metadata_type_loads(llama):
         llama.gguf_inspect(blob[:-1])
 
 
+def test_gguf_parser_survives_hostile_counts_and_shapes(llama):
+    """A short file must not be able to reserve memory through an array count, a shape whose byte count
+    wraps 64 bits must not pass the size check, and a row that is not a whole number of blocks is refused at
+    parse time (the row dequantizers and the device kernels walk rows block by block)."""
+    def s(x):
+        return struct.pack("<Q", len(x)) + x
+
+    def gguf(kv_bytes, n_kv, tensor_bytes, n_tensors, data=b""):
+        head = b"GGUF" + struct.pack("<Iqq", 3, n_tensors, n_kv) + kv_bytes + tensor_bytes
+        pad = (len(head) + 31) // 32 * 32 - len(head)
+        return np.frombuffer(head + b"\0" * pad + data, dtype=np.uint8)
+
+    # array of 2^40 one-byte elements in a 60-byte file; and of 2^40 strings
+    for elem in (0, 8):
+        kv = s(b"a.arr") + struct.pack("<i", 9) + struct.pack("<iQ", elem, 1 << 40)
+        with pytest.raises(llama.LlamaError, match="truncated"):
+            llama.gguf_inspect(gguf(kv, 1, b"", 0))
+    # a count that fits the remaining bytes but whose elements do not
+    kv = s(b"a.arr") + struct.pack("<i", 9) + struct.pack("<iQ", 10, 3) + struct.pack("<Q", 1)
+    with pytest.raises(llama.LlamaError, match="truncated"):
+        llama.gguf_inspect(gguf(kv, 1, b"", 0))
+    # F32 tensor of 2^62 elements: 2^64 bytes wraps to 0
+    t = s(b"t") + struct.pack("<Iqq", 2, 1 << 31, 1 << 31) + struct.pack("<iQ", 0, 0)
+    with pytest.raises(llama.LlamaError, match="bad shape|truncated"):
+        llama.gguf_inspect(gguf(b"", 0, t, 1))
+    # element count beyond 64 bits
+    t = s(b"t") + struct.pack("<Iqqq", 3, 1 << 40, 1 << 40, 1 << 40) + struct.pack("<iQ", 0, 0)
+    with pytest.raises(llama.LlamaError, match="bad shape"):
+        llama.gguf_inspect(gguf(b"", 0, t, 1))
+    # Q8_0 rows of 48 columns: two rows make whole blocks in total (96 = 3 x 32), one row does not
+    t = s(b"t") + struct.pack("<Iqq", 2, 48, 2) + struct.pack("<iQ", 8, 0)
+    with pytest.raises(llama.LlamaError, match="bad shape"):
+        llama.gguf_inspect(gguf(b"", 0, t, 1, b"\0" * 102))
+    t = s(b"t") + struct.pack("<Iqq", 2, 64, 2) + struct.pack("<iQ", 8, 0)
+    assert llama.gguf_inspect(gguf(b"", 0, t, 1, b"\0" * 136)) == (1, 0, 32)
+
+
 # ------------------------------------------------------------------ building blocks
 
 def test_row_dequantizers_match_the_oracle_bit_for_bit(llama, pkg):
