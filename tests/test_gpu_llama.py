@@ -152,3 +152,36 @@ def test_mixtral_shaped_routed_layer_matches_the_cpu_path(pkg, llama, tmp_path):
     # one token alone takes the single-token kernels for its two experts: same row up to summation order
     alone = gpu.moe_ffn(0, x[5:6])
     assert np.all(np.abs(alone[0].astype(np.float64) - want[5]) <= 1e-4 * np.maximum(np.abs(want[5]), rms / 4))
+
+
+def test_config4_full_size_greedy_decode_on_every_path(pkg, llama, tmp_path):
+    """Benchmark configuration 4 at full size: a random Llama-3-8B-shaped model (32 layers, d 4096, 32 query /
+    8 K/V heads of 128, ffn 14336, vocab 128256, RMSNorm eps 1e-5, RoPE base 5e5, Q4_K blocks with a Q6_K head),
+    128 random prompt ids as one batch, then 128 greedy single-token steps over a paged K/V cache with blocks of
+    16 positions.  The device-resident session, the host session (one GPU round trip per product, the
+    reference's call structure) and the same host code over the restated AVX2 kernels of the reference's CPU
+    path must produce the same 129 tokens.  The smallest gap between the two largest logits of any step,
+    relative to the largest logit, says how much room rounding differences had (langtax/src/decode.rs:12104-12114
+    takes the first maximum, so a flip needs two logits closer than the paths' disagreement, about 1e-5)."""
+    path = tmp_path / "llama3_8b_shape.gguf"
+    llama.write_synthetic_llama(path, n_layer=32, n_embd=4096, n_head=32, n_head_kv=8, n_ff=14336, n_vocab=128256,
+                                rope_base=5e5, rms_eps=1e-5, weight_std=0.02, seed=20240531)
+    prompt = np.random.default_rng(20240531).integers(0, 128256, 128)
+    gpu = llama.Llama(path=path)
+    host_toks, _, _ = gpu.session(kv_block=16).generate_greedy(prompt, 129)
+    dev_toks, _, _ = gpu.session(kv_block=16, device_positions=256).generate_greedy(prompt, 129)
+    gpu.close()
+    cpu = llama.Llama(path=path, products=llama.CALLBACK, matmul=cpu_products(True, 0))
+    s = cpu.session(kv_block=16)
+    logits = s.forward(prompt)
+    cpu_toks, gaps = [], []
+    for step in range(129):
+        top2 = np.partition(logits, -2)[-2:]
+        gaps.append(float(top2[1] - top2[0]) / float(np.abs(logits).max()))
+        cpu_toks.append(llama.argmax(logits))
+        if step < 128:
+            logits = s.forward([cpu_toks[-1]])
+    print(f"\nconfig 4: 129 tokens, smallest top-2 logit gap {min(gaps):.3e} of the largest logit (step {int(np.argmin(gaps))})")
+    assert host_toks.tolist() == cpu_toks, int(np.sum(np.cumprod(host_toks == np.array(cpu_toks))))
+    assert dev_toks.tolist() == cpu_toks, int(np.sum(np.cumprod(dev_toks == np.array(cpu_toks))))
+    assert min(gaps) > 1e-5

@@ -424,7 +424,7 @@ def test_config3_batched_gemm(pkg, gpu, ty, rows, cols):
     w = _baseline_matrix(ty, rows, cols, rng)
     m = gpu.upload_packed(ty, rows, cols, w)
     rb = K.row_bytes(ty, cols)
-    sample = np.unique(np.concatenate([[0, 1, rows - 1], rng.integers(0, rows, 29)]))
+    sample = _edge_rows(rows, rng, 12)
     w_sample = np.concatenate([w[r * rb:(r + 1) * rb] for r in sample])
     x_all = rng.normal(0, 1, 512 * cols).astype(np.float32)
     for tokens in (1, 8, 32, 128, 512):
@@ -443,6 +443,20 @@ def test_config3_batched_gemm(pkg, gpu, ty, rows, cols):
             _, mag0 = O.gemm_f64_mag(ty, cols, 1, w_sample, x[:cols], sample.size)
             assert np.all(np.abs(y2[0, sample].astype(np.float64) - y1[sample]) <= 2 * K.single_kernel_bound(cols, mag0[0]))
     m.close()
+
+
+def _edge_rows(rows, rng, n_random):
+    """Rows to hold against the oracle when a product is too large to check whole: both sides of every kind
+    of boundary the multi-token kernels have (16- and 32-row matrix-core sets, the 64 rows of a wavefront,
+    the 256-row tile of a workgroup) at the start, in the middle and at the end of the matrix, plus a few
+    random ones."""
+    fixed = [0, 1, 15, 16, 17, 31, 32, 33, 63, 64, 65, 255, 256, 257]
+    mid = (rows // 2) // 256 * 256
+    fixed += [mid - 1, mid, mid + 63, mid + 64]
+    last = (rows - 1) // 256 * 256
+    fixed += [last - 1, last, last + 1, rows - 65, rows - 64, rows - 33, rows - 17, rows - 2, rows - 1]
+    picks = np.concatenate([np.array(fixed), rng.integers(0, rows, n_random)])
+    return np.unique(picks[(picks >= 0) & (picks < rows)])
 
 
 def test_config5_expert_grouped_gemm(pkg, gpu):
@@ -464,7 +478,7 @@ def test_config5_expert_grouped_gemm(pkg, gpu):
         y = np.full(sum(tokens) * rows, np.nan, np.float32)
         gpu.gemm_grouped(mats, tokens, x_packed, y)
         rb = K.row_bytes(K.Q4_K, cols)
-        sample = np.unique(np.concatenate([[0, rows - 1], rng.integers(0, rows, 14)]))
+        sample = _edge_rows(rows, rng, 4)
         yo = 0
         for e in range(n_exp):
             ye = y[yo:yo + tokens[e] * rows].reshape(tokens[e], rows)

@@ -110,6 +110,49 @@ def test_q5_0_pack_bytes_known_answer():
     assert O.vec_dot_row(K.Q5_0, 32, w, x, simd=True) == np.float32(10.5)
 
 
+def test_q5_1_pack_bytes_known_answer():
+    """langtax/src/quant.rs:11028-11046: the reference's byte-level answers for a Q5_1 block, and its
+    dot against values decoded here from those bytes (numpy float16), not by the oracle's dequantizer."""
+    qs = np.zeros(32, np.uint8)
+    qs[0], qs[16], qs[7], qs[23] = 19, 28, 7, 15
+    w = O.pack_q5_1_block(25.0 / 100.0, 5.0 / 100.0, qs)
+    assert w.size == 24
+    assert w[8] == 0xc3                                   # low nibble y[0] = 19, high nibble y[16] = 28
+    qh = int(w[4:8].view(np.uint32)[0])
+    assert qh & 0x00010001 == 0x00010001                  # their fifth bits
+    assert w[15] == 0xf7                                  # low nibble y[7] = 7, high nibble y[23] = 15
+    assert qh & ((1 << 7) | (1 << 23)) == 0
+    d, m = (float(v) for v in w[0:4].view(np.float16))
+    assert d == 0.25 and abs(m - 0.05) < 2 ** -14 and m <= 0.05   # the encoder rounds toward zero
+    x = np.zeros(32, np.float32)
+    x[0], x[16], x[7], x[23] = 2.0, 4.0, 1.0, 3.0
+    codes = np.zeros(32)
+    codes[[0, 16, 7, 23]] = 19, 28, 7, 15
+    expected = float(np.sum((codes * d + m) * x))
+    for simd in (False, True):
+        got = float(O.vec_dot_row(K.Q5_1, 32, w, x, simd=simd))
+        assert abs(got - expected) / (1 + abs(expected)) < 1e-5
+    row = O.dequant(K.Q5_1, 32, w, 1)[0]
+    assert row.tolist() == (np.float32(codes) * np.float32(d) + np.float32(m)).tolist()   # two roundings, no FMA
+
+
+def test_q4_0_low_and_high_nibbles_are_elements_j_and_j_plus_16():
+    """langtax/src/gguf.rs:1130-1137: v[0] = 1, v[16] = 2 packed at scale 1 against x[0] = 3, x[16] = 4
+    gives 11 (a kernel that read the nibbles as neighbours x[2j], x[2j+1] would give 3)."""
+    v = np.zeros(32, np.int8)
+    v[0], v[16] = 1, 2
+    w = O.pack_q4_0_block(1.0, v)
+    assert w[0:2].view(np.float16)[0] == 1.0
+    assert w[2] == 0xa9                                   # (1 + 8) | (2 + 8) << 4
+    assert np.all(w[3:] == 0x88)                          # zero codes carry the bias 8 in both nibbles
+    x = np.zeros(32, np.float32)
+    x[0], x[16] = 3.0, 4.0
+    assert O.vec_dot_row(K.Q4_0, 32, w, x) == np.float32(11.0)
+    assert O.vec_dot_row(K.Q4_0, 32, w, x, simd=True) == np.float32(11.0)
+    row = O.dequant(K.Q4_0, 32, w, 1)[0]
+    assert row[0] == 1.0 and row[16] == 2.0 and np.count_nonzero(row) == 2
+
+
 def test_q4_k_scale_pack_round_trip_all_values():
     """Every 6-bit scale/min through pack -> scale_min_k4 (quant.rs:4852-4878, 8901-8912)."""
     rng = np.random.default_rng(7)
