@@ -127,8 +127,9 @@ int lnh_gemm_shared(lnh_exec *exec, size_t n_mats, const lnh_matrix *const *mats
  * through the host (native-cuda/src/gpu.rs:301-303, 332-334).
  * Products of three or more tokens by a quantized matrix use a workspace that
  * belongs to the executor and grows on demand (growing allocates, so it cannot
- * happen while `stream` is being captured into a graph: run the largest shape
- * once before capturing; a workspace that captured launches point at stays
+ * happen while `stream` is being captured into a graph: such a call fails with
+ * LNH_ERR_INVALID before anything is launched - run the largest shape once
+ * before capturing; a workspace that captured launches point at stays
  * allocated until the executor is destroyed, also after a later call has
  * made the executor move to a larger one).  Calls of one executor must therefore be enqueued on
  * one stream at a time; calls that overlap on different streams race on it. */

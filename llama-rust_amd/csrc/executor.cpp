@@ -141,8 +141,17 @@ bool ensure_pinned(lnh_exec *e, size_t in_floats, size_t out_floats) {
 // goes: a caller may have captured launches that point at it into a HIP graph (a decode step that is replayed
 // while another call, a longer prompt say, makes the workspace grow), and work already queued may still use
 // it.  Growth is by at least half, so everything retired together is smaller than twice the live buffer.
-int ensure_workspace(lnh_exec *e, size_t bytes) {
+int ensure_workspace(lnh_exec *e, hipStream_t s, size_t bytes) {
     if (bytes <= e->ws_cap) return LNH_OK;
+    // Growing allocates, which a stream under capture cannot record: refuse before anything is launched
+    // instead of leaving the caller with a broken capture.
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (s && hipStreamIsCapturing(s, &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone)
+        return fail(e, LNH_ERR_INVALID,
+                    "the multi-token workspace must grow to " + std::to_string(bytes) +
+                        " bytes while the stream is being captured: run the largest product once before capturing, "
+                        "or use lnh_gemm_device_noalloc");
+    (void)hipGetLastError();
     size_t want = bytes > e->ws_cap + e->ws_cap / 2 ? bytes : e->ws_cap + e->ws_cap / 2;
     want += want / 4;
     void *fresh = nullptr;
@@ -169,7 +178,7 @@ int launch_products(lnh_exec *e, hipStream_t s, size_t n, const lnh_matrix *cons
         tiled[g] = mats[g]->tiled;
         toks[g] = (uint32_t)tokens[g];
     }
-    int rc = ensure_workspace(e, nh::gemm_workspace_bytes(views.data(), toks.data(), (uint32_t)n));
+    int rc = ensure_workspace(e, s, nh::gemm_workspace_bytes(views.data(), toks.data(), (uint32_t)n));
     if (rc != LNH_OK) return rc;
     hipError_t h = nh::launch_gemm_groups(s, views.data(), tiled.data(), toks.data(), xs, ys, (uint32_t)n, e->d_ws, e->ws_cap);
     if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");

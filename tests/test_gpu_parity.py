@@ -18,6 +18,7 @@ dequantized weights:
         as e -> 0 for ANY f32 summation order, the reference's CPU kernels
         included, because the rounding error scales with sum|w x|, not with |e|).
 """
+import importlib
 import os
 
 import numpy as np
@@ -229,6 +230,53 @@ def test_invalid_operations_preserve_output_with_a_live_device(pkg):
         again = np.zeros(1, np.float32)
         pkg.gemv(fmt.ty, fmt.cols, packed, x, again)  # still usable, same answer
         assert again[0] == ok[0]
+
+
+def test_workspace_growth_under_stream_capture_is_refused_not_recorded(pkg):
+    """A multi-token product whose workspace does not exist yet cannot be captured into a HIP graph (growing
+    allocates): the call fails with nothing launched and the capture stays usable.  The allocation-free entry
+    point can be captured at once, and the ordinary one after one eager call; replays of both equal the eager
+    result bit for bit."""
+    hip = importlib.import_module("llama-rust_amd.hiprt")
+    g = pkg.HipGemv(0)  # a fresh executor: no workspace yet
+    rng = np.random.default_rng(31)
+    rows, cols, tokens = 512, 1024, 8
+    w = K.random_packed(K.Q4_K, rows, cols, rng, signed=False, scale=0.02)
+    m = g.upload_packed(K.Q4_K, rows, cols, w)
+    x = rng.normal(0, 1, tokens * cols).astype(np.float32)
+    xd = hip.DeviceBuffer.from_numpy(x)
+    ya, yb, yc = (hip.DeviceBuffer(tokens * rows * 4) for _ in range(3))
+    stream = hip.Stream()
+    seen = {}
+
+    def enqueue(s):
+        try:
+            g.gemm_device(m, tokens, xd.ptr, ya.ptr, s.ptr)
+        except pkg.NativeHipError as e:
+            seen["code"], seen["text"] = e.code, str(e)
+        g.gemm_device_noalloc(m, tokens, xd.ptr, yb.ptr, s.ptr)
+
+    graph = hip.Graph(stream, enqueue)
+    assert seen.get("code") == pkg.ERR_INVALID and "being captured" in seen["text"]
+    g.gemm_device(m, tokens, xd.ptr, yc.ptr, stream.ptr)   # eager: grows the workspace
+    stream.synchronize()
+    want = yc.to_numpy(np.float32)
+    check(want, K.Q4_K, cols, tokens, rows, w, x, "eager product before the replays")
+    graph2 = hip.Graph(stream, lambda s: g.gemm_device(m, tokens, xd.ptr, ya.ptr, s.ptr))   # now it can be captured
+    for _ in range(3):
+        yb.fill_byte(0xff)
+        ya.fill_byte(0xff)
+        graph.launch()
+        graph2.launch()
+        stream.synchronize()
+        assert np.array_equal(yb.to_numpy(np.float32).view(np.uint32), want.view(np.uint32))
+        assert np.array_equal(ya.to_numpy(np.float32).view(np.uint32), want.view(np.uint32))
+    graph.destroy()
+    graph2.destroy()
+    for b in (xd, ya, yb, yc):
+        b.free()
+    m.close()
+    g.close()
 
 
 def test_q4k_matrix_beyond_32_bit_plane_offsets_is_refused(pkg, gpu):
