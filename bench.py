@@ -40,13 +40,36 @@ sys.path.insert(0, ROOT)
 METRIC = "Q4_K/Q8_0 GEMV HBM GB/s (% of peak); 8B-shape decode tok/s, batch 1"
 HBM_PEAK_GBS = 8000.0
 BF16_MFMA_PEAK_TFLOPS = 2500.0
-# HBM bytes per Q4_K launch over algorithmic bytes, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this script (counters scaled by a 1 GiB copy kernel: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the
-# figures and commands are in profiles/decode_gemv_q4k_q6k_8b_step.txt.  Not measured by this run.
-Q4K_TRAFFIC_OVER_ALGORITHMIC = 1.0089
+# HBM bytes per Q4_K launch over algorithmic bytes come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# script (counters scaled by a 1 GiB copy kernel), summarised in the file below; a run of this script cannot
+# read the counters itself.  The summary names the kernel source it was taken with (a SHA-256 of the .inc file);
+# when that no longer matches the source in the tree, the figure is stale and `traffic` is reported as null.
+TRAFFIC_PROFILE = os.path.join("profiles", "decode_gemv_q4k_q6k_8b_step.txt")
+KERNEL_SOURCE = os.path.join("llama-rust_amd", "csrc", "gemv_kernels.inc")
+
+
+def profiled_traffic():
+    """{'ratio': measured HBM bytes / algorithmic bytes of the Q4_K launches or None, 'source': where from}."""
+    import hashlib
+    import re
+    try:
+        text = open(os.path.join(ROOT, TRAFFIC_PROFILE)).read()
+        ratio = float(re.search(r"^traffic_over_algorithmic_q4k:\s*([0-9.]+)", text, re.M).group(1))
+        profiled = re.search(r"^kernel_source_sha256:\s*([0-9a-f]{64})", text, re.M).group(1)
+        now = hashlib.sha256(open(os.path.join(ROOT, KERNEL_SOURCE), "rb").read()).hexdigest()
+    except (OSError, AttributeError, ValueError) as e:
+        return {"ratio": None, "source": f"{TRAFFIC_PROFILE} unreadable ({type(e).__name__})"}
+    if profiled != now:
+        return {"ratio": None, "source": f"{TRAFFIC_PROFILE} was taken with another {KERNEL_SOURCE} "
+                                         f"(sha256 {profiled[:12]}, now {now[:12]}): stale, re-profile"}
+    return {"ratio": ratio, "source": f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, {TRAFFIC_PROFILE} (kernel source sha256 {now[:12]})"}
+
+
 Q4_0, Q5_0, Q5_1, Q8_0, Q4_K, Q6_K = 2, 6, 7, 8, 12, 14
+F32, F16 = 0, 1
 BLOCK = {Q4_0: (32, 18, 0), Q5_0: (32, 22, 0), Q5_1: (32, 24, 0), Q8_0: (32, 34, 0), Q4_K: (256, 144, 0),
-         Q6_K: (256, 210, 208)}  # columns, bytes, offset of d
+         Q6_K: (256, 210, 208), F16: (1, 2, 0), F32: (1, 4, 0)}  # columns, bytes, offset of d
+FP32_PEAK_TFLOPS = 157.3
 N_LAYERS, D, D_KV, FF, VOCAB = 32, 4096, 1024, 14336, 128256
 # (name, rows, cols, which activation buffer it reads).  Products that read the same buffer are
 # independent of each other (q/k/v of the normed hidden state, gate/up of the normed residual);
@@ -73,6 +96,9 @@ def algorithmic_bytes(ty, rows, cols, tokens=1):
 
 def synth_matrix(ty, rows, cols, rng):
     """Packed GGUF bytes: uniform random codes / 6-bit scales, |N(0, 0.02)| f16 super-block scales."""
+    if ty in (F16, F32):
+        w = rng.normal(0, 0.02, (rows, cols)).astype(np.float16 if ty == F16 else np.float32)
+        return w.view(np.uint8).reshape(-1)
     qk, bb, d_off = BLOCK[ty]
     nb = cols // qk
     blk = rng.integers(0, 256, size=(rows, nb, bb), dtype=np.uint8)
@@ -80,6 +106,36 @@ def synth_matrix(ty, rows, cols, rng):
     blk[:, :, d_off:d_off + 2 * n_scales] = (np.abs(rng.normal(0, 0.02, (rows, nb, n_scales))).astype(np.float16)
                                              .view(np.uint8).reshape(rows, nb, 2 * n_scales))
     return blk.reshape(-1)
+
+
+# Layers of the step whose matrices the CPU baseline sweeps: 8 x 123 MB + a sixteenth of the head = 1.0 GB per
+# sweep, beyond any last-level cache, so the figure is a memory-streaming one like the GPU's.
+CPU_SAMPLE_LAYERS = 8
+
+
+def host_cpu():
+    """Model name, physical cores and logical CPUs of this host, and whether a Rust toolchain is present (with
+    one the reference's own `--no-default-features --features simd` build could be timed instead of the port)."""
+    import shutil
+    model, cores = "unknown", set()
+    try:
+        phys = core = None
+        for line in open("/proc/cpuinfo"):
+            key, _, val = line.partition(":")
+            key, val = key.strip(), val.strip()
+            if key == "model name":
+                model = val
+            elif key == "physical id":
+                phys = val
+            elif key == "core id":
+                core = val
+            elif not key and phys is not None and core is not None:
+                cores.add((phys, core))
+                phys = core = None
+    except OSError:
+        pass
+    return {"cpu_model": model, "physical_cores": len(cores) or None, "logical_cpus": os.cpu_count(),
+            "cargo_present": shutil.which("cargo") is not None}
 
 
 def cpu_baseline(sample, x_by_cols, seconds):
@@ -102,10 +158,13 @@ def cpu_baseline(sample, x_by_cols, seconds):
         dt = time.perf_counter() - t0
         if dt >= seconds or n >= 2000:
             break
-    return {"value": nbytes * n / dt / 1e9, "unit": "GB/s", "cores": int(threads), "kind": "port",
-            "sample": f"layer 0 (7 Q4_K GEMVs) + first {sample[-1][1]} rows of the Q6_K head, "
-                      f"{nbytes / 1e6:.1f} MB per sweep, {n} sweeps in {dt:.1f} s, AVX2 port of the reference simd kernels",
-            "tok_per_s_equiv": n / dt * nbytes / TOKEN_BYTES}
+    out = {"value": nbytes * n / dt / 1e9, "unit": "GB/s", "cores": int(threads), "kind": "port",
+           "sample": f"the first {CPU_SAMPLE_LAYERS} layers (7 Q4_K GEMVs each) + first {sample[-1][1]} rows of the Q6_K head, "
+                     f"{nbytes / 1e6:.1f} MB per sweep, {n} sweeps in {dt:.1f} s, AVX2 port of the reference simd kernels",
+           "cache_resident": False,
+           "tok_per_s_equiv": n / dt * nbytes / TOKEN_BYTES}
+    out.update(host_cpu())
+    return out
 
 
 def timed_us(hip, stream, enqueue, n_variants, reps):
@@ -196,6 +255,29 @@ def other_workloads(pkg, hip, gpu, stream, rng, cpu):
                 m.close()
             xd.free(); yd.free()
 
+    # F16 and F32 weights, 4096x14336 (the two dtypes whose products never reach the matrix cores: one token on the
+    # streaming GEMV kernel, more on a vector-ALU tile kernel)
+    for ty, nm in ((F16, "f16"), (F32, "f32")):
+        rows, cols, n = D, FF, 4
+        ws = [synth_matrix(ty, rows, cols, rng) for _ in range(n)]
+        ms = [gpu.upload_packed(ty, rows, cols, w) for w in ws]
+        x = rng.normal(0, 1, 512 * cols).astype(np.float32)
+        xd, yd = hip.DeviceBuffer.from_numpy(x), hip.DeviceBuffer(512 * rows * 4)
+        for tokens in (1, 8, 128, 512):
+            us = timed_us(hip, stream, lambda i: gpu.gemm_device(ms[i], tokens, xd.ptr, yd.ptr, stream.ptr), n, 3)
+            gpu.gemm_device(ms[0], tokens, xd.ptr, yd.ptr, stream.ptr); stream.synchronize()
+            check(f"{nm} GEMM {rows}x{cols} M={tokens}", ty, rows, cols, tokens, ws[0], x[:tokens * cols], yd)
+            flops = 2.0 * rows * cols * tokens
+            out[f"gemm_{nm}_{rows}x{cols}_m{tokens}"] = {
+                "call_us": round(us, 2), "tflops": round(flops / us / 1e6, 1),
+                "fp32_frac": round(flops / us / 1e6 / FP32_PEAK_TFLOPS, 4) if tokens > 1 else None,
+                "weight_gbs": round(rows * row_bytes(ty, cols) / us / 1e3, 1),
+                "hbm_frac": round(algorithmic_bytes(ty, rows, cols, tokens) / us / 1e3 / HBM_PEAK_GBS, 4),
+                "bound": "fp32" if tokens >= 128 else "hbm", "cpu_us": None}
+        for m in ms:
+            m.close()
+        xd.free(); yd.free()
+
     # one MoE projection: 8 Q4_K experts 4096 -> 14336, 16 tokens each, one grouped call
     n_exp, per = 8, 16
     sets = 2  # two sets of experts = 528 MB, so that no call is served from the Infinity Cache
@@ -256,6 +338,40 @@ def other_workloads(pkg, hip, gpu, stream, rng, cpu):
         for ms_ in group:
             for m in ms_:
                 m.close()
+    xd.free(); hd_.free(); gd.free(); ud.free(); yd2.free()
+
+    # The same layer as the reference runs it, routing included (langtax/src/decode.rs:9938-10292): a Mixtral-shaped
+    # layer of a synthetic GGUF, 64 tokens through the host code - router product, softmax, top-2, grouping, the
+    # three grouped expert products with their host round trips, SiLU * up and the weighted scatter on the host.
+    import tempfile
+    L = importlib.import_module("llama-rust_amd.llama")
+    with tempfile.TemporaryDirectory() as tmp:
+        path = os.path.join(tmp, "mixtral_layer.gguf")
+        L.write_synthetic_llama(path, n_layer=1, n_embd=D, n_head=32, n_head_kv=8, n_ff=FF, n_vocab=256, block_type=Q4_K,
+                                embd_type=Q8_0, output_type=Q8_0, seed=8, n_expert=n_exp, n_expert_used=2)
+        model = L.Llama(path=path)
+        xt = rng.normal(0, 1, (n_tok, D)).astype(np.float32)
+        got = model.moe_ffn(0, xt)  # uploads the experts
+        t0 = time.perf_counter()
+        reps = 5
+        for _ in range(reps):
+            got = model.moe_ffn(0, xt)
+        host_us = (time.perf_counter() - t0) / reps * 1e6
+        entry = {"call_us": round(host_us, 1), "tokens": n_tok, "experts": n_exp, "top_k": 2,
+                 "scope": "whole routed feed-forward through the host seam: 4 GPU calls with host round trips + host routing, SiLU*up, scatter"}
+        if cpu:
+            ref = L.Llama(path=path, products=L.CALLBACK,
+                          matmul=lambda ty, n_rows, n_cols, n_tokens, w, x: O.gemm(ty, n_cols, n_tokens, w, x, n_rows, simd=True, threads=0))
+            t0 = time.perf_counter()
+            want = ref.moe_ffn(0, xt)
+            entry["cpu_us"] = round((time.perf_counter() - t0) * 1e6, 1)
+            rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+            if not np.all(np.abs(got.astype(np.float64) - want) <= 1e-4 * np.maximum(np.abs(want), rms / 4)):
+                raise RuntimeError("routed MoE layer: GPU route disagrees with the CPU path")
+            entry["matches_cpu_path"] = True
+            ref.close()
+        model.close()
+        out["moe_layer_routed_host_seam_q4_k_8_experts_top2_64_tokens"] = entry
     return out
 
 
@@ -322,7 +438,23 @@ def greedy_decode(pkg, layers, check_cpu, seed):
             c = L.Llama(path=path, products=L.CALLBACK,
                         matmul=lambda ty, n_rows, n_cols, n_tokens, w, x:
                         O.gemm(ty, n_cols, n_tokens, w, x, n_rows, simd=True, threads=0))
-            ctoks, cp, cd = c.session(kv_block=16).generate_greedy(prompt, 129)
+            # step by step, so that every step's logits are seen: the smallest gap between the two largest logits
+            # (relative to the largest logit) is the room rounding differences between the paths had
+            cs = c.session(kv_block=16)
+            t0 = time.perf_counter()
+            logits = cs.forward(prompt)
+            cp = time.perf_counter() - t0
+            ctoks, gaps = [], []
+            t0 = time.perf_counter()
+            for step in range(129):
+                top2 = np.partition(logits, -2)[-2:]
+                gaps.append(float(top2[1] - top2[0]) / float(np.abs(logits).max()))
+                ctoks.append(L.argmax(logits))
+                if step < 128:
+                    logits = cs.forward([ctoks[-1]])
+            cd = time.perf_counter() - t0
+            ctoks = np.array(ctoks, dtype=toks.dtype)
+            out.update(min_top2_logit_gap=float(f"{min(gaps):.3e}"), min_top2_logit_gap_step=int(np.argmin(gaps)))
             same = int(np.sum(np.cumprod(toks == ctoks)))
             out.update(cpu_prefill_s=round(cp, 2), cpu_decode_tok_per_s=round(128 / cd, 3), cpu_threads=O.load().lro_worker_count(D),
                        tokens_identical=bool(same == 129), identical_prefix=same)
@@ -379,7 +511,7 @@ def main():
             if (slot, name) not in y_bufs:
                 y_bufs[(slot, name)] = hip.DeviceBuffer(rows * 4)
             ys.append(y_bufs[(slot, name)].ptr)
-            if layer == 0:
+            if layer < CPU_SAMPLE_LAYERS:
                 sample.append((Q4_K, rows, cols, w, src))
         if layer % 8 == 7:
             log(f"[bench] uploaded {layer + 1}/{args.layers} layers ({time.perf_counter() - t_setup:.1f} s)")
@@ -397,18 +529,67 @@ def main():
     head_batch = gpu.make_batch([head], [1], [x_dev["h1"].ptr], [head_y.ptr])
     enqueue_layers = lambda s=stream: gpu.gemm_batch_device(layers_batch, s.ptr)
     enqueue_head = lambda s=stream: gpu.gemm_batch_device(head_batch, s.ptr)
-    enqueue_layers(); enqueue_head(); stream.synchronize()       # first launches configure the kernels
+
+    def enqueue_step(s=stream):
+        enqueue_layers(s)
+        enqueue_head(s)
+
+    # The launches of one shape across all layers, for the per-shape figures: [q,k,v] [o] [gate,up] [down].
+    shape_groups = {"[q,k,v]": ("q", "k", "v"), "[o]": ("o",), "[gate,up]": ("gate", "up"), "[down]": ("down",)}
+    names = [nm for nm, _, _, _ in LAYER]
+    # A launch's time is taken inside the real chain, as the difference between the whole chain and the chain
+    # without that shape's launches: a chain of one shape alone would replay 0.3-0.45 GB of matrices, most of
+    # which the 256 MB Infinity Cache would then serve.
+    shape_batches, shape_bytes = {}, {}
+    for label, members in shape_groups.items():
+        idx = [layer * len(LAYER) + k for layer in range(args.layers) for k, nm in enumerate(names) if nm not in members]
+        shape_batches[label] = gpu.make_batch([mats[i] for i in idx], [1] * len(idx), [xs[i] for i in idx], [ys[i] for i in idx])
+        shape_bytes[label] = sum(algorithmic_bytes(Q4_K, r, c) for nm, r, c, _ in LAYER if nm in members)
+    enqueue_step(); stream.synchronize()       # first launches configure the kernels
+    for b in shape_batches.values():
+        gpu.gemm_batch_device(b, stream.ptr)
+    stream.synchronize()
+
+    # The yardstick: a kernel that only reads, at the byte counts of the step's launches, chained the same way,
+    # over memory of its own (4.4 GB, so nothing comes from the Infinity Cache either).
+    read_sizes = [shape_bytes[k] // 16 * 16 for k in ("[q,k,v]", "[o]", "[gate,up]", "[down]")]
+    head_bytes = algorithmic_bytes(Q6_K, VOCAB, D)
+    read_buf = hip.DeviceBuffer(args.layers * sum(read_sizes) + head_bytes // 16 * 16)
+    read_buf.fill_byte(0x5a)
+
+    def enqueue_read_step(s=stream, without=None, head=True):
+        at = read_buf.ptr
+        for _ in range(args.layers):
+            for k, nbytes in enumerate(read_sizes):
+                if without != k:
+                    gpu.calibration_read(at, nbytes, s.ptr)
+                at += nbytes
+        if head:
+            gpu.calibration_read(at, head_bytes // 16 * 16, s.ptr)
+
+    enqueue_read_step(); stream.synchronize()
+
     if not args.no_graph:
-        g_layers = hip.Graph(stream, enqueue_layers)
-        g_head = hip.Graph(stream, enqueue_head)
-        run_layers, run_head = g_layers.launch, g_head.launch
+        graphs = {"step": hip.Graph(stream, enqueue_step), "layers": hip.Graph(stream, enqueue_layers),
+                  "head": hip.Graph(stream, enqueue_head), "read_step": hip.Graph(stream, enqueue_read_step)}
+        for label, b in shape_batches.items():
+            graphs[label] = hip.Graph(stream, lambda s, b=b: gpu.gemm_batch_device(b, s.ptr))
+        graphs["read layers"] = hip.Graph(stream, lambda s: enqueue_read_step(s, head=False))
+        for k, label in enumerate(shape_groups):
+            graphs["read " + label] = hip.Graph(stream, lambda s, k=k: enqueue_read_step(s, without=k, head=False))
+        run = {k: g.launch for k, g in graphs.items()}
     else:
-        run_layers, run_head = enqueue_layers, enqueue_head
+        run = {"step": enqueue_step, "layers": enqueue_layers, "head": enqueue_head, "read_step": enqueue_read_step}
+        for label, b in shape_batches.items():
+            run[label] = lambda b=b: gpu.gemm_batch_device(b, stream.ptr)
+        run["read layers"] = lambda: enqueue_read_step(stream, head=False)
+        for k, label in enumerate(shape_groups):
+            run["read " + label] = lambda k=k: enqueue_read_step(stream, without=k, head=False)
 
     # sanity: a sample of layer-0 outputs against the CPU oracle before timing anything
     import oracle as O
-    run_layers(); run_head(); stream.synchronize()
-    for (ty, rows, cols, w, src), (name, _, _, _) in zip(sample, LAYER):
+    run["step"](); stream.synchronize()
+    for (ty, rows, cols, w, src), (name, _, _, _) in zip(sample[:len(LAYER)], LAYER):
         got = y_bufs[(0, name)].to_numpy(np.float32)[:64]
         want = O.gemm_f64(ty, cols, 1, w[:64 * row_bytes(ty, cols)], x_host[src], 64)[0]
         if not np.allclose(got, want, rtol=1e-4, atol=1e-4 * float(np.sqrt(np.mean(want ** 2)))):
@@ -423,34 +604,59 @@ def main():
         stream.synchronize()
         src.free(); dst.free()
 
+    def replay_us(key, reps):
+        """Mean microseconds of one replay of run[key], from HIP events on the launch stream around `reps`
+        back-to-back replays."""
+        run[key](); stream.synchronize()
+        a, b = hip.Event(), hip.Event()
+        a.record(stream)
+        for _ in range(reps):
+            run[key]()
+        b.record(stream)
+        stream.synchronize()
+        return a.elapsed_ms(b) * 1e3 / reps
+
     for _ in range(args.warmup):
-        run_layers(); run_head()
+        run["step"]()
     stream.synchronize()
 
-    ev = [(hip.Event(), hip.Event(), hip.Event()) for _ in range(args.steps)]
+    # The timed region: K steps, each one graph of all 129 launches, between two synchronisations.
+    a_ev, b_ev = hip.Event(), hip.Event()
     hip.device_synchronize()
     t0 = time.perf_counter()
-    for a, b, c in ev:
-        a.record(stream)
-        run_layers()
-        b.record(stream)
-        run_head()
-        c.record(stream)
+    a_ev.record(stream)
+    for _ in range(args.steps):
+        run["step"]()
+    b_ev.record(stream)
     stream.synchronize()
     hip.device_synchronize()
     wall = time.perf_counter() - t0
+    step_event_ms = a_ev.elapsed_ms(b_ev) / args.steps
 
-    q4k_ms = sum(a.elapsed_ms(b) for a, b, _ in ev)
-    head_ms = sum(b.elapsed_ms(c) for _, b, c in ev)
+    # The same launches again, the Q4_K part and the head on their own (HIP events on the launch stream).
+    q4k_ms = replay_us("layers", args.steps) / 1e3
+    head_ms = replay_us("head", args.steps) / 1e3
     q4k_bytes = (args.layers * sum(algorithmic_bytes(Q4_K, r, c) for _, r, c, _ in LAYER))
     n_launch = args.layers * LAUNCHES_PER_LAYER
-    head_bytes = algorithmic_bytes(Q6_K, VOCAB, D)
     step_bytes = q4k_bytes + head_bytes
     ms_per_step = wall * 1e3 / args.steps
     value = step_bytes / (wall / args.steps) / 1e9
-    q4k_launch_us = q4k_ms * 1e3 / (args.steps * n_launch)
-    q4k_gbs = q4k_bytes / (q4k_ms / args.steps * 1e-3) / 1e9
-    head_gbs = head_bytes / (head_ms / args.steps * 1e-3) / 1e9
+    q4k_launch_us = q4k_ms * 1e3 / n_launch
+    q4k_gbs = q4k_bytes / (q4k_ms * 1e-3) / 1e9
+    head_gbs = head_bytes / (head_ms * 1e-3) / 1e9
+
+    # Per launch shape, and the read-only yardstick at the same sizes (mean over the layers' launches).
+    per_shape = {}
+    reps = max(3, args.steps // 2)
+    layers_us, read_layers_us = replay_us("layers", reps), replay_us("read layers", reps)
+    for k, label in enumerate(shape_groups):
+        us = (layers_us - replay_us(label, reps)) / args.layers
+        read_us = (read_layers_us - replay_us("read " + label, reps)) / args.layers
+        per_shape[label] = {"bytes": shape_bytes[label], "launch_us": round(us, 2),
+                            "achieved": round(shape_bytes[label] / us / 1e3, 1), "frac": round(shape_bytes[label] / us / 1e3 / HBM_PEAK_GBS, 4),
+                            "plain_read_us": round(read_us, 2), "frac_of_plain_read": round(read_us / us, 3)}
+    read_step_us = replay_us("read_step", max(3, args.steps // 2))
+    traffic = profiled_traffic()
 
     out = {
         "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -459,20 +665,30 @@ def main():
         "config": {"workload": f"Llama-3-8B decode GEMV, batch 1: {args.layers} layers x 7 Q4_K products + Q6_K head 4096->128256",
                    "weights_gb": round(step_bytes / 1e9, 3), "products_per_step": n_q4k + 1, "launches_per_step": n_launch + 1,
                    "launch_grouping": "per layer [q,k,v] [o] [gate,up] [down]: products sharing an input are one launch",
-                   "launch_mode": "eager" if args.no_graph else "hip_graph"},
+                   "launch_mode": "eager" if args.no_graph else "one hip_graph per step (layers and head)"},
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "tok_per_s": round(args.steps / wall, 1),
         "tok_per_s_scope": "the timed step: the weight products of one token; decode_tok_per_s_end_to_end is a whole greedy decode",
+        "ms_per_step_hip_events": round(step_event_ms, 4),
         "roofline": {"bound": "hbm", "kernel": "gemv_q4k_kernel", "achieved": round(q4k_gbs, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(q4k_gbs / HBM_PEAK_GBS, 4),
-                     "traffic": round(Q4K_TRAFFIC_OVER_ALGORITHMIC * q4k_bytes / n_launch),
-                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiles/decode_gemv_q4k_q6k_8b_step.txt",
+                     "traffic": round(traffic["ratio"] * q4k_bytes / n_launch) if traffic["ratio"] else None,
+                     "traffic_source": traffic["source"],
                      "bytes_per_launch": round(q4k_bytes / n_launch), "launch_us": round(q4k_launch_us, 3),
-                     "launches_timed": args.steps * n_launch},
+                     "launches_timed": args.steps * n_launch,
+                     "timing": "HIP events on the launch stream around K back-to-back replays of the graph of the 128 Q4_K launches, right after the timed region",
+                     "per_shape": per_shape,
+                     "per_shape_method": "time of the 128-launch chain minus the chain without that shape's 32 launches, per launch; plain_read_us the same for a kernel that only reads",
+                     "plain_read_same_sizes": {
+                         "what": "a kernel that only reads, launched as the same chain at the same byte counts (4 per layer + head)",
+                         "step_us": round(read_step_us, 1), "gbs": round(step_bytes / read_step_us / 1e3, 1),
+                         "frac_of_peak": round(step_bytes / read_step_us / 1e3 / HBM_PEAK_GBS, 4),
+                         "this_step_vs_plain_read": round(read_step_us / (ms_per_step * 1e3), 3)}},
         "other_kernels": {"gemv_q6k_kernel (head)": {"achieved": round(head_gbs, 1), "unit": "GB/s",
                                                      "frac": round(head_gbs / HBM_PEAK_GBS, 4),
-                                                     "launch_us": round(head_ms * 1e3 / args.steps, 2)}},
+                                                     "launch_us": round(head_ms * 1e3, 2)}},
     }
+    read_buf.free()
     for m in mats:
         m.close()
     head.close()

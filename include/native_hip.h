@@ -185,6 +185,11 @@ int lnh_gemv_swiglu_device(lnh_exec *exec, const lnh_matrix *gate, const lnh_mat
 /* Measurement aid, no counterpart in the reference: a plain device-to-device copy kernel
  * (nbytes a multiple of 16) whose known traffic calibrates HBM byte counters. */
 int lnh_calibration_copy(lnh_exec *exec, void *device_dst, const void *device_src, size_t nbytes, void *stream);
+/* Measurement aid, no counterpart in the reference: a kernel that reads nbytes (a multiple of 16, at least 32)
+ * of device memory once, requested the way the single-token kernels request their weights, and does nothing
+ * with them.  Its duration at the sizes of a decode step's launches is the ceiling those launches are held
+ * against beside the 8 TB/s figure. */
+int lnh_calibration_read(lnh_exec *exec, const void *device_src, size_t nbytes, void *stream);
 /* Block the host until everything enqueued on the executor's own stream is done. */
 int lnh_synchronize(lnh_exec *exec);
 

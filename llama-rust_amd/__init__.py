@@ -110,6 +110,7 @@ def load_library():
         "lnh_gemv_fused_device": (C.c_int, [vp, sz, pvp, vp, pvp, C.c_int, C.c_int, vp, C.c_float, vp]),
         "lnh_gemv_swiglu_device": (C.c_int, [vp, vp, vp, vp, vp, C.c_int, vp, C.c_float, vp]),
         "lnh_calibration_copy": (C.c_int, [vp, vp, vp, sz, vp]),
+        "lnh_calibration_read": (C.c_int, [vp, vp, sz, vp]),
         "lnh_synchronize": (C.c_int, [vp]),
         "lnh_shape_checked": (C.c_int, [sz, sz, sz, sz, C.POINTER(u32), C.POINTER(u32)]),
         "lnh_validate": (C.c_int, [vp, sz, vp, sz]),
@@ -364,6 +365,9 @@ class HipGemv:
     def calibration_copy(self, dst_ptr, src_ptr, nbytes, stream=0):
         self._check(self._lib.lnh_calibration_copy(self._h, C.c_void_p(dst_ptr), C.c_void_p(src_ptr), nbytes,
                                                    C.c_void_p(stream)))
+
+    def calibration_read(self, src_ptr, nbytes, stream=0):
+        self._check(self._lib.lnh_calibration_read(self._h, C.c_void_p(src_ptr), nbytes, C.c_void_p(stream)))
 
     def synchronize(self):
         self._check(self._lib.lnh_synchronize(self._h))

@@ -695,6 +695,18 @@ int lnh_calibration_copy(lnh_exec *e, void *device_dst, const void *device_src, 
     return LNH_OK;
 }
 
+int lnh_calibration_read(lnh_exec *e, const void *device_src, size_t nbytes, void *stream) {
+    if (!e) return LNH_ERR_INVALID;
+    if (!device_src || nbytes % 16 != 0 || nbytes == 16) return fail(e, LNH_ERR_INVALID, "read needs a device pointer and a multiple of 16 bytes, at least 32");
+    hipError_t h = hipSetDevice(e->ctx->device);
+    if (h != hipSuccess) return hip_fail(e, h, "hipSetDevice");
+    const int rc = ensure_scratch(e, 0, 1);  // the kernel's never-written sink
+    if (rc != LNH_OK) return rc;
+    h = nh::launch_read(stream ? static_cast<hipStream_t>(stream) : e->stream, device_src, nbytes, e->d_out);
+    if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
+    return LNH_OK;
+}
+
 int lnh_synchronize(lnh_exec *e) {
     if (!e) return LNH_ERR_INVALID;
     hipError_t h = hipStreamSynchronize(e->stream);

@@ -64,6 +64,9 @@ void *static_scratch(int device);
 
 // dst[0, nbytes) = src[0, nbytes) (nbytes a multiple of 16): reference traffic for counter calibration.
 hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t nbytes);
+// Reads src[0, nbytes) once and writes nothing (sink: any 4 writable device bytes, never written in practice):
+// the streaming-read yardstick the single-token kernels are measured against.
+hipError_t launch_read(hipStream_t stream, const void *src, size_t nbytes, void *sink);
 // The same copy with a grid sized by nbytes: activations between pinned host staging memory (which the
 // device reads and writes directly) and device scratch, a few KB at a time.
 hipError_t launch_copy_small(hipStream_t stream, void *dst, const void *src, size_t nbytes);

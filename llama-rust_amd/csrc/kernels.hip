@@ -718,6 +718,32 @@ hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t nb
     return hipGetLastError();
 }
 
+// Plain streaming read: every thread requests eight consecutive-by-256 16-byte pieces at once and the
+// grid covers the whole range in one go, like the single-token kernels' weight loads; nothing is written
+// (the store is behind a condition that never holds).  What this takes is what the memory system gives
+// a reader that does no arithmetic at all.
+__global__ __launch_bounds__(256) void read_kernel(const uint4 *__restrict__ p, size_t n16, uint32_t *sink) {
+    uint4 v[8];
+    const size_t base = (size_t)blockIdx.x * 8 * 256 + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const size_t i = base + (size_t)k * 256;
+        v[k] = p[i < n16 ? i : 0];
+    }
+    uint32_t a = 0;
+#pragma unroll
+    for (int k = 0; k < 8; k++) a ^= v[k].x ^ v[k].y ^ v[k].z ^ v[k].w;
+    if (a == 0x9e3779b9u && n16 == 1) *sink = a;
+}
+
+hipError_t launch_read(hipStream_t stream, const void *src, size_t nbytes, void *sink) {
+    const size_t n16 = nbytes / 16;
+    if (n16 == 0) return hipSuccess;
+    hipLaunchKernelGGL(read_kernel, dim3((unsigned)((n16 + 2047) / 2048)), dim3(256), 0, stream,
+                       static_cast<const uint4 *>(src), n16, static_cast<uint32_t *>(sink));
+    return hipGetLastError();
+}
+
 hipError_t launch_copy_small(hipStream_t stream, void *dst, const void *src, size_t nbytes) {
     const size_t n16 = nbytes / 16, want = (n16 + 255) / 256, most = (size_t)g_cu_count * 8;
     if (n16 == 0) return hipSuccess;

@@ -105,7 +105,7 @@ def test_every_extern_declaration_matches_the_header():
                    "lnh_gemm_device_noalloc"):
         assert needed in r, needed
     # measurement and test helpers of the header are deliberately left out of the binding
-    assert set(c) - set(r) <= {"lnh_calibration_copy", "lnq_parse_cache_bytes", "lnq_automatic_cache_bytes",
+    assert set(c) - set(r) <= {"lnh_calibration_copy", "lnh_calibration_read", "lnq_parse_cache_bytes", "lnq_automatic_cache_bytes",
                                "lnq_admission_requires_eviction", "lnq_cache_stats", "lnq_reset"}
 
 
