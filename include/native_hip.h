@@ -79,9 +79,12 @@ int lnh_upload_f32(lnh_exec *exec, size_t rows, size_t cols, const float *weight
  * F32 at langtax/src/quant.rs:6746-6755 followed by upload (native_gpu.rs:190-194).
  * `nbytes` must equal rows * row_bytes(type, cols); cols must be a whole number
  * of blocks (32 for Q4_0/Q5_0/Q5_1/Q8_0, 256 for Q4_K/Q6_K).
- * A quantized matrix is kept twice, in two layouts: one the single-token
- * kernels stream, one the multi-token (matrix-core) kernels stream, so it takes
- * about twice its GGUF size in HBM (lnh_matrix_info reports the exact figure). */
+ * A quantized matrix has two layouts in HBM: the one the single-token kernels
+ * stream is made here; the one the multi-token (matrix-core) kernels stream is
+ * made from it by the first product of three or more tokens (or by
+ * lnh_matrix_prepare), so a matrix that only ever meets one token at a time
+ * (an output head, an embedding table) takes its GGUF size once, the others
+ * about twice (lnh_matrix_info reports the figure as it stands). */
 int lnh_upload_packed(lnh_exec *exec, uint32_t ggml_type, size_t rows, size_t cols, const uint8_t *bytes,
                       size_t nbytes, lnh_matrix **out);
 /* Same, from bytes that already sit in device memory of this executor's GPU. */
@@ -89,8 +92,16 @@ int lnh_upload_packed_device(lnh_exec *exec, uint32_t ggml_type, size_t rows, si
                              const void *device_bytes, size_t nbytes, lnh_matrix **out);
 /* Drop of a CudaMatrix.  Safe after its executor was destroyed. */
 void lnh_matrix_free(lnh_matrix *matrix);
+/* device_bytes: what the matrix holds in HBM now (it grows once, when the multi-token layout is made). */
 int lnh_matrix_info(const lnh_matrix *matrix, uint32_t *ggml_type, size_t *rows, size_t *cols,
                     size_t *device_bytes);
+/* Makes now whatever products of up to max_tokens tokens by this matrix will need beyond the upload (the
+ * multi-token layout when max_tokens >= 3 and the dtype is quantized): allocates, runs on the executor's own
+ * stream and returns when the copy is complete.  For callers that will run such products where allocating is
+ * not possible: inside a stream capture (a product that finds the layout missing there fails with
+ * LNH_ERR_INVALID before anything is launched) or through lnh_gemm_device_noalloc.  No counterpart in the
+ * reference, whose resident form is one F32 array. */
+int lnh_matrix_prepare(lnh_exec *exec, const lnh_matrix *matrix, size_t max_tokens);
 
 /* ------------------------------------------------------------------ products (host buffers) */
 
@@ -143,7 +154,9 @@ int lnh_gemm_grouped_device(lnh_exec *exec, size_t n_groups, const lnh_matrix *c
  * array inside the library's device code (LNH_NOALLOC_WORKSPACE_BYTES per GPU, held from lnh_create on
  * that GPU until the process ends) instead of the executor's grow-on-demand allocation: the call
  * never allocates or frees.  A product that needs more fails with LNH_ERR_INVALID
- * (the message states the need) before anything is launched.  Every call on one GPU, from any executor, uses the
+ * (the message states the need) before anything is launched; so does a product of three or more tokens by a
+ * quantized matrix whose multi-token layout has not been made yet (lnh_matrix_prepare, or any earlier such product
+ * through an allocating entry point, makes it).  Every call on one GPU, from any executor, uses the
  * same array and nothing in it outlives a call: calls that may overlap on one GPU (different streams,
  * different threads) race on it and must be ordered by the caller. */
 #define LNH_NOALLOC_WORKSPACE_BYTES ((size_t)64 << 20)

@@ -97,6 +97,7 @@ def load_library():
         "lnh_upload_packed_device": (C.c_int, [vp, u32, sz, sz, vp, sz, pvp]),
         "lnh_matrix_free": (None, [vp]),
         "lnh_matrix_info": (C.c_int, [vp, C.POINTER(u32), psz, psz, psz]),
+        "lnh_matrix_prepare": (C.c_int, [vp, vp, sz]),
         "lnh_gemv": (C.c_int, [vp, vp, vp, sz, vp, sz]),
         "lnh_gemm": (C.c_int, [vp, vp, sz, vp, sz, vp, sz]),
         "lnh_gemv_once": (C.c_int, [vp, vp, sz, vp, sz, vp, sz]),
@@ -318,6 +319,11 @@ class HipGemv:
     def gemm_device(self, matrix, tokens, x_ptr, y_ptr, stream=0):
         self._check(self._lib.lnh_gemm_device(self._h, matrix._h, tokens, C.c_void_p(x_ptr), C.c_void_p(y_ptr),
                                               C.c_void_p(stream)))
+
+    def prepare(self, matrix, max_tokens):
+        """Makes now what products of up to max_tokens tokens by this matrix need beyond the upload (the multi-token
+        layout of a quantized matrix), for callers that will run them where nothing may be allocated."""
+        self._check(self._lib.lnh_matrix_prepare(self._h, matrix._h, max_tokens))
 
     def gemm_device_noalloc(self, matrix, tokens, x_ptr, y_ptr, stream=0):
         """gemm_device with the library's fixed device workspace: never allocates (include/native_hip.h)."""

@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <cstring>
 #include <memory>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -34,7 +35,13 @@ struct lnh_matrix {
     void *dev = nullptr;
     size_t dev_bytes = 0;
     nh::MatView view{};   // planes the single-token kernels read
-    nh::MatView tiled{};  // row-interleaved copy the multi-token kernels read (quantized dtypes)
+    // Row-interleaved copy the multi-token kernels read (quantized dtypes).  Made from the planes by the first
+    // product that needs it (or lnh_matrix_prepare), so that a matrix only ever used with one token (an output
+    // head, an embedding table) is resident once.  p0 is null until then.
+    mutable std::mutex lazy;
+    mutable void *dev_tiled = nullptr;
+    mutable size_t tiled_bytes = 0;
+    mutable nh::MatView tiled{};
 };
 
 struct lnh_exec {
@@ -168,6 +175,51 @@ int ensure_workspace(lnh_exec *e, hipStream_t s, size_t bytes) {
     return LNH_OK;
 }
 
+// The tiled copy of m, made now if no product has needed it yet.  Making it allocates, which a stream under capture
+// cannot record, and the copy must be complete before any stream reads it: the one-time build is followed by a
+// synchronisation of the building stream.
+int ensure_tiled(lnh_exec *e, hipStream_t s, const lnh_matrix *m) {
+    std::lock_guard<std::mutex> lock(m->lazy);
+    if (m->tiled.p0) return LNH_OK;
+    const nh::TiledSpec ts = nh::tiled_spec(m->view.type, m->view.rows, m->view.cols);
+    if (ts.total == 0) return LNH_OK;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (s && hipStreamIsCapturing(s, &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone)
+        return fail(e, LNH_ERR_INVALID,
+                    "the matrix has no multi-token copy yet and the stream is being captured: call lnh_matrix_prepare (or run one "
+                    "multi-token product) before capturing");
+    (void)hipGetLastError();
+    hipError_t h = hipSetDevice(m->ctx->device);
+    if (h != hipSuccess) return hip_fail(e, h, "hipSetDevice");
+    void *dev = nullptr;
+    h = hipMalloc(&dev, ts.total);
+    if (h != hipSuccess) return hip_fail(e, h, "HIP matrix allocation (multi-token copy)");
+    uint8_t *tb = static_cast<uint8_t *>(dev);
+    nh::MatView t = m->view;
+    t.p0 = tb + ts.offset[0];
+    t.p1 = tb + ts.offset[1];
+    t.p2 = tb + ts.offset[2];
+    t.p3 = tb + ts.offset[3];
+    t.s0 = (uint32_t)ts.per_row[0];
+    t.s1 = (uint32_t)ts.per_row[1];
+    t.s2 = (uint32_t)ts.per_row[2];
+    t.s3 = (uint32_t)ts.per_row[3];
+    hipStream_t bs = s ? s : e->stream;
+    // rows that pad the last tile are decoded like any other and then dropped: give them defined bytes
+    h = hipMemsetAsync(tb, 0, ts.total, bs);
+    if (h == hipSuccess) h = nh::launch_retile(bs, t, m->view);
+    const hipError_t hs = hipStreamSynchronize(bs);
+    if (h == hipSuccess) h = hs;
+    if (h != hipSuccess) {
+        (void)hipFree(dev);
+        return hip_fail(e, h, "HIP matrix re-layout (multi-token copy)");
+    }
+    m->dev_tiled = dev;
+    m->tiled_bytes = ts.total;
+    m->tiled = t;
+    return LNH_OK;
+}
+
 // Launch n products; xs/ys are device pointers.
 int launch_products(lnh_exec *e, hipStream_t s, size_t n, const lnh_matrix *const *mats, const size_t *tokens,
                     const float *const *xs, float *const *ys) {
@@ -175,8 +227,12 @@ int launch_products(lnh_exec *e, hipStream_t s, size_t n, const lnh_matrix *cons
     std::vector<uint32_t> toks(n);
     for (size_t g = 0; g < n; g++) {
         views[g] = mats[g]->view;
-        tiled[g] = mats[g]->tiled;
         toks[g] = (uint32_t)tokens[g];
+        if (nh::product_reads_tiled(views[g].type, toks[g]) && views[g].rows != 0) {
+            const int rt = ensure_tiled(e, s, mats[g]);
+            if (rt != LNH_OK) return rt;
+        }
+        tiled[g] = mats[g]->tiled;
     }
     int rc = ensure_workspace(e, s, nh::gemm_workspace_bytes(views.data(), toks.data(), (uint32_t)n));
     if (rc != LNH_OK) return rc;
@@ -188,11 +244,10 @@ int launch_products(lnh_exec *e, hipStream_t s, size_t n, const lnh_matrix *cons
 int make_matrix(lnh_exec *e, uint32_t type, size_t rows, size_t cols, const void *src, bool src_on_device,
                 size_t nbytes, lnh_matrix **out) {
     nh::PlaneSpec ps = nh::plane_spec(type, rows, cols);
-    nh::TiledSpec ts = nh::tiled_spec(type, rows, cols);
     hipError_t h = hipSetDevice(e->ctx->device);
     if (h != hipSuccess) return hip_fail(e, h, "hipSetDevice");
     void *dev = nullptr;
-    h = hipMalloc(&dev, ps.total + ts.total);
+    h = hipMalloc(&dev, ps.total);
     if (h != hipSuccess) return hip_fail(e, h, "HIP matrix allocation");
     void *staging = nullptr;
     const void *src_dev = src;
@@ -208,7 +263,7 @@ int make_matrix(lnh_exec *e, uint32_t type, size_t rows, size_t cols, const void
     auto m = std::make_unique<lnh_matrix>();
     m->ctx = e->ctx;
     m->dev = dev;
-    m->dev_bytes = ps.total + ts.total;
+    m->dev_bytes = ps.total;
     uint8_t *base = static_cast<uint8_t *>(dev);
     m->view.p0 = base + ps.offset[0];
     m->view.p1 = base + ps.offset[1];
@@ -222,21 +277,6 @@ int make_matrix(lnh_exec *e, uint32_t type, size_t rows, size_t cols, const void
     m->view.rows = (uint32_t)rows;
     m->view.cols = (uint32_t)cols;
     m->view.nb = (uint32_t)(cols / nh::block_elems(type));
-    if (ts.total != 0) {
-        uint8_t *tb = base + ps.total;
-        m->tiled = m->view;
-        m->tiled.p0 = tb + ts.offset[0];
-        m->tiled.p1 = tb + ts.offset[1];
-        m->tiled.p2 = tb + ts.offset[2];
-        m->tiled.p3 = tb + ts.offset[3];
-        m->tiled.s0 = (uint32_t)ts.per_row[0];
-        m->tiled.s1 = (uint32_t)ts.per_row[1];
-        m->tiled.s2 = (uint32_t)ts.per_row[2];
-        m->tiled.s3 = (uint32_t)ts.per_row[3];
-        // rows that pad the last tile are decoded like any other and then dropped: give them defined bytes
-        if (h == hipSuccess) h = hipMemsetAsync(tb, 0, ts.total, e->stream);
-        if (h == hipSuccess) h = nh::launch_repack_tiled(e->stream, m->tiled, src_dev);
-    }
     if (h == hipSuccess) h = nh::launch_repack(e->stream, m->view, src_dev);
     hipError_t hs = hipStreamSynchronize(e->stream);
     if (h == hipSuccess) h = hs;
@@ -347,7 +387,10 @@ int lnh_create(int device_ordinal, lnh_exec **out) {
         return fail(nullptr, LNH_ERR_DEVICE, std::string("kernels are built for gfx950 only, device is ") + prop.gcnArchName);
     size_t lds = prop.sharedMemPerBlockOptin ? prop.sharedMemPerBlockOptin : prop.sharedMemPerBlock;
     if (lds > 80 * 1024) lds = 80 * 1024;  // two workgroups per CU must fit in the 160 KB LDS
-    nh::set_device_limits(prop.multiProcessorCount, lds);
+    if (!nh::set_device_limits(prop.multiProcessorCount, lds))
+        return fail(nullptr, LNH_ERR_DEVICE,
+                    "HIP device " + std::to_string(device_ordinal) + " differs from the GPU this process already runs on (compute units or LDS per "
+                    "workgroup): one kind of GPU per process");
     auto e = std::make_unique<lnh_exec>();
     e->ctx = std::make_shared<Ctx>();
     e->ctx->device = device_ordinal;
@@ -355,12 +398,18 @@ int lnh_create(int device_ordinal, lnh_exec **out) {
     h = hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking);
     if (h != hipSuccess) return hip_fail(nullptr, h, "hipStreamCreate");
     float unit = 0.f;
-    h = nh::probe_fp8_nibble_unit(e->stream, &unit);
+    bool bf16_exact = false, i4_exact = false;
+    h = nh::probe_nibble_converts(e->stream, &unit, &bf16_exact, &i4_exact);
     if (h != hipSuccess) {
         (void)hipStreamDestroy(e->stream);
-        return hip_fail(nullptr, h, "fp8 unpack probe");
+        return hip_fail(nullptr, h, "nibble convert probe");
     }
-    nh::set_fp8_nibble_unit(unit);
+    if (!nh::set_nibble_converts(unit, bf16_exact, i4_exact)) {
+        (void)hipStreamDestroy(e->stream);
+        return fail(nullptr, LNH_ERR_DEVICE,
+                    "HIP device " + std::to_string(device_ordinal) + " converts nibble bytes differently from the GPU this process already runs on: "
+                    "one kind of GPU per process");
+    }
     // address of this device's copy of the static workspace (lnh_gemm_device_noalloc), looked up while
     // the device is current
     h = nh::static_scratch_init(device_ordinal);
@@ -435,7 +484,17 @@ void lnh_matrix_free(lnh_matrix *m) {
     if (!m) return;
     (void)hipSetDevice(m->ctx->device);
     if (m->dev) (void)hipFree(m->dev);
+    if (m->dev_tiled) (void)hipFree(m->dev_tiled);
     delete m;
+}
+
+int lnh_matrix_prepare(lnh_exec *e, const lnh_matrix *m, size_t max_tokens) {
+    if (!e) return LNH_ERR_INVALID;
+    if (!m) return fail(e, LNH_ERR_INVALID, "HIP matrix is null");
+    if (m->ctx.get() != e->ctx.get()) return fail(e, LNH_ERR_FOREIGN, "HIP matrix belongs to a different executor");
+    if (max_tokens > UINT32_MAX) return fail(e, LNH_ERR_INVALID, "GEMM tokens exceed u32");
+    if (!nh::product_reads_tiled(m->view.type, (uint32_t)max_tokens)) return LNH_OK;
+    return ensure_tiled(e, e->stream, m);
 }
 
 int lnh_matrix_info(const lnh_matrix *m, uint32_t *type, size_t *rows, size_t *cols, size_t *device_bytes) {
@@ -443,7 +502,10 @@ int lnh_matrix_info(const lnh_matrix *m, uint32_t *type, size_t *rows, size_t *c
     if (type) *type = m->view.type;
     if (rows) *rows = m->view.rows;
     if (cols) *cols = m->view.cols;
-    if (device_bytes) *device_bytes = m->dev_bytes;
+    if (device_bytes) {
+        std::lock_guard<std::mutex> lock(m->lazy);
+        *device_bytes = m->dev_bytes + m->tiled_bytes;  // the multi-token copy counts once it exists
+    }
     return LNH_OK;
 }
 
@@ -554,6 +616,12 @@ int lnh_gemm_device_noalloc(lnh_exec *e, const lnh_matrix *m, size_t tokens, con
                     "product needs " + std::to_string(need) + " bytes of workspace, the allocation-free entry point holds " +
                         std::to_string(nh::STATIC_SCRATCH_BYTES) + ": use lnh_gemm_device or fewer tokens per call");
     hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
+    if (nh::product_reads_tiled(m->view.type, tok32)) {
+        std::lock_guard<std::mutex> lock(m->lazy);
+        if (!m->tiled.p0)
+            return fail(e, LNH_ERR_INVALID,
+                        "the matrix has no multi-token copy yet and this entry point does not allocate: call lnh_matrix_prepare first");
+    }
     const hipError_t h = nh::launch_gemm_groups(s, &m->view, &m->tiled, &tok32, &dx, &dy, 1, ws, nh::STATIC_SCRATCH_BYTES);
     if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
     return LNH_OK;

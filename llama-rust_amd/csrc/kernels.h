@@ -6,19 +6,22 @@
 
 namespace nh {
 
-// CU count and the largest dynamic LDS a workgroup may ask for on this device.
-void set_device_limits(int cu_count, size_t lds_per_block);
+// CU count and the largest dynamic LDS a workgroup may ask for on this device.  Held once per process: the
+// first call sets them, a later call returns false when its values differ (the caller refuses the executor).
+bool set_device_limits(int cu_count, size_t lds_per_block);
 
-// Value the fp8 (E4M3) unpack gives for byte 0x01 on this device when bytes 0..15 decode
-// linearly (n * unit), else 0: nibble kernels then take the byte-convert path.
-void set_fp8_nibble_unit(float unit);
-// Runs a 16-thread probe kernel and reports that unit (0 when the decode is not linear).
-hipError_t probe_fp8_nibble_unit(hipStream_t stream, float *unit_out);
+// What the device's converts give for nibble bytes: the value of byte 0x01 under the fp8 (E4M3) unpack when bytes
+// 0..15 decode linearly (n * unit, a power of two), else 0 (nibble kernels then take the byte-convert path);
+// whether the packed fp8 -> bf16 convert with scale 512 gives the integers 0..15; whether the signed 4-bit
+// convert with a byte select gives (n - 8) / 16.  Probed by a 16-thread kernel, held once per process like the limits.
+hipError_t probe_nibble_converts(hipStream_t stream, float *unit_out, bool *bf16_out, bool *i4_out);
+bool set_nibble_converts(float unit, bool bf16_exact, bool i4_exact);
 
 // Scatter the GGUF bytes at src_device (device memory) into the planes of m.
 hipError_t launch_repack(hipStream_t stream, const MatView &m, const void *src_device);
-// Same for the tiled copy (matview.h); tiled.s0..s3 hold the units per row of each plane.
-hipError_t launch_repack_tiled(hipStream_t stream, const MatView &tiled, const void *src_device);
+// The tiled copy (matview.h) from the planes of the same matrix, both on the device; tiled.s0..s3 hold the units
+// per row of each plane.
+hipError_t launch_retile(hipStream_t stream, const MatView &tiled, const MatView &planes);
 
 // y[t, r] = sum_c W[r, c] x[t, c]; x and y are device pointers, token-major.
 // Products of three or more tokens by a quantized matrix run on the matrix cores (two tokens: two

@@ -31,9 +31,17 @@ static bool g_nibble_i4 = false;    // the signed 4-bit convert with a byte sele
 static int g_cu_count = 256;
 static size_t g_lds_limit = 64 * 1024;
 
-void set_device_limits(int cu_count, size_t lds_per_block) {
-    if (cu_count > 0) g_cu_count = cu_count;
-    if (lds_per_block > 0) g_lds_limit = lds_per_block;
+// The launchers' view of the device is held once per process.  Every executor reports what it found on its
+// device; the first report sets it, a later one that differs is refused by the caller (one kind of GPU per
+// process: a second kind would need these per device).
+static bool g_limits_set = false;
+bool set_device_limits(int cu_count, size_t lds_per_block) {
+    if (cu_count <= 0 || lds_per_block == 0) return false;
+    if (g_limits_set) return cu_count == g_cu_count && lds_per_block == g_lds_limit;
+    g_cu_count = cu_count;
+    g_lds_limit = lds_per_block;
+    g_limits_set = true;
+    return true;
 }
 
 // Jobs must share x, dtype and column count.  hipErrorInvalidValue = "does not fit this
@@ -113,7 +121,7 @@ __global__ void fp8_nibble_probe(float *out) {
     out[128 + 8 * threadIdx.x + 7] = i4_of_byte<3>(hi_n >> 4);
 }
 
-hipError_t probe_fp8_nibble_unit(hipStream_t stream, float *unit_out) {
+hipError_t probe_nibble_converts(hipStream_t stream, float *unit_out, bool *bf16_out, bool *i4_out) {
     *unit_out = 0.f;
     float *d = nullptr;
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&d), 256 * sizeof(float));
@@ -136,16 +144,26 @@ hipError_t probe_fp8_nibble_unit(hipStream_t stream, float *unit_out) {
     bool exact = true;  // fp8 -> bf16 with scale 512 must give the integers 0..15
     for (int n = 0; n < 16; n++)
         for (int k = 0; k < 4; k++) exact = exact && h[64 + 4 * n + k] == (float)n;
-    g_nibble_bf16 = exact;
+    const bool bf16_exact = exact;
     exact = true;
     for (int n = 0; n < 16; n++)
         for (int k = 0; k < 8; k++) exact = exact && h[128 + 8 * n + k] == (float)(n - 8) / 16.0f;
-    g_nibble_i4 = exact;
+    if (bf16_out) *bf16_out = bf16_exact;
+    if (i4_out) *i4_out = exact;
     return hipSuccess;
 }
 
 static float g_nib_mul = 0.f;  // 1 / (value of fp8 byte 0x01); 0 = fp8 unpack not usable
-void set_fp8_nibble_unit(float unit) { g_nib_mul = unit > 0.f ? 1.0f / unit : 0.f; }
+static bool g_converts_set = false;
+bool set_nibble_converts(float unit, bool bf16_exact, bool i4_exact) {
+    const float mul = unit > 0.f ? 1.0f / unit : 0.f;
+    if (g_converts_set) return mul == g_nib_mul && bf16_exact == g_nibble_bf16 && i4_exact == g_nibble_i4;
+    g_nib_mul = mul;
+    g_nibble_bf16 = bf16_exact;
+    g_nibble_i4 = i4_exact;
+    g_converts_set = true;
+    return true;
+}
 
 template <int LB, int NW, int PL, int PRO>
 static hipError_t launch_q4k_lb(hipStream_t stream, const GemvBatch &b, uint32_t units, size_t lds) {
@@ -625,7 +643,6 @@ static hipError_t launch_plain(hipStream_t stream, const MatView &m, uint32_t to
 // Length of the run of groups starting at g that one MFMA launch can take.
 // (Two tokens are two single-token launches: 2 x 9-15 us on the 33-44 MB matrices against 24-29 us for the
 // three launches of the MFMA path, and row t of the result is then bit for bit the GEMV of token t.)
-constexpr uint32_t MM_MIN_TOKENS = 3;
 static uint32_t mm_run(const MatView *mats, const uint32_t *tokens, uint32_t n, uint32_t g) {
     if (!mm_type(mats[g].type) || tokens[g] < MM_MIN_TOKENS) return 0;
     uint32_t run = 1;

@@ -164,6 +164,13 @@ inline PlaneSpec plane_spec(uint32_t t, size_t rows, size_t cols) {
 // (code units in the order of the GGUF block).  F32/F16 have no such copy.
 constexpr uint32_t TILE_ROWS = 256;
 
+// Products of at least this many tokens by a quantized matrix run on the matrix cores and read the tiled copy
+// (two tokens are two single-token launches).
+constexpr uint32_t MM_MIN_TOKENS = 3;
+inline bool product_reads_tiled(uint32_t t, uint32_t tokens) {
+    return tokens >= MM_MIN_TOKENS && t != T_F32 && t != T_F16 && type_supported(t);
+}
+
 struct TiledSpec {
     size_t unit[4], per_row[4];
     size_t offset[4];

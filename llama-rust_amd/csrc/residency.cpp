@@ -164,9 +164,29 @@ void commit(State &s, Pending &p) {
     p.keep = false;
 }
 
+// After a product: a cached matrix that made its multi-token layout in this product (matview.h) is charged for
+// it from now on; what then exceeds the budget leaves from the front, the matrix just used last of all.
+void recharge(State &s, const lnh_matrix *m) {
+    for (Entry &en : s.cache) {
+        if (en.matrix->m != m) continue;
+        size_t dev = 0;
+        if (lnh_matrix_info(m, nullptr, nullptr, nullptr, &dev) != LNH_OK) return;
+        const size_t now = dev + en.packed.size();
+        if (now > en.bytes) {
+            s.bytes += now - en.bytes;
+            en.bytes = now;
+        }
+        break;
+    }
+    while (!s.cache.empty() && s.bytes > s.limit) {
+        s.bytes = s.bytes > s.cache.front().bytes ? s.bytes - s.cache.front().bytes : 0;
+        s.cache.pop_front();
+    }
+}
+
 // Resident matrix for these bytes: hit -> move to back, miss -> evict from the
 // front until it fits, upload packed; `pending` then holds the entry to keep if within budget.
-int resident(State &s, uint32_t type, size_t rows, size_t cols, const uint8_t *w, size_t w_len,
+int resident(State &s, uint32_t type, size_t rows, size_t cols, size_t n_tokens, const uint8_t *w, size_t w_len,
              std::shared_ptr<Holder> *out, Pending *pending) {
     WeightKey key = make_key(type, rows, cols, w, w_len);
     for (size_t i = 0; i < s.cache.size(); i++) {
@@ -181,9 +201,15 @@ int resident(State &s, uint32_t type, size_t rows, size_t cols, const uint8_t *w
         }
     }
     s.misses++;
-    // both device copies of the matrix (matview.h) plus the host copy kept for the identity check
-    size_t bytes = nh::plane_spec(type, rows, cols).total + nh::tiled_spec(type, rows, cols).total + w_len;
+    // what the matrix will hold on the device after this product (the single-token layout, plus the multi-token
+    // layout when this product makes it: matview.h) and the host copy kept for the identity check
+    size_t bytes = nh::plane_spec(type, rows, cols).total + w_len;
     if (bytes < w_len) return qfail(LNH_ERR_INVALID, "resident matrix size overflow");
+    if (nh::product_reads_tiled(type, n_tokens > UINT32_MAX ? UINT32_MAX : (uint32_t)n_tokens)) {
+        const size_t more = nh::tiled_spec(type, rows, cols).total;
+        if (bytes + more < bytes) return qfail(LNH_ERR_INVALID, "resident matrix size overflow");
+        bytes += more;
+    }
     while (!s.cache.empty() && admission_requires_eviction(s.bytes, bytes, s.limit)) {
         s.bytes = s.bytes > s.cache.front().bytes ? s.bytes - s.cache.front().bytes : 0;
         s.cache.pop_front();
@@ -240,11 +266,12 @@ int lnq_gemm(uint32_t type, size_t n_cols, size_t n_tokens, const uint8_t *w, si
     BusyGuard guard(&s);
     std::shared_ptr<Holder> mat;
     Pending pending;
-    rc = resident(s, type, n_rows, n_cols, w, w_len, &mat, &pending);
+    rc = resident(s, type, n_rows, n_cols, n_tokens, w, w_len, &mat, &pending);
     if (rc != LNH_OK) return rc;
     rc = lnh_gemm(s.gpu, mat->m, n_tokens, x, x_len, y, y_len);
     if (rc != LNH_OK) return qfail(rc, lnh_last_error(s.gpu));
     commit(s, pending);
+    recharge(s, mat->m);
     return LNH_OK;
 }
 
@@ -293,7 +320,7 @@ int lnq_gemm_grouped(uint32_t type, size_t n_cols, size_t n_rows, size_t n_group
         if (toks[g] == 0) continue;
         // parts uploaded earlier in this call are not in the cache yet: a part that repeats is uploaded again,
         // which costs time, never correctness
-        rc = resident(s, type, n_rows, n_cols, parts[g], part_len, &holders[g], &pending[g]);
+        rc = resident(s, type, n_rows, n_cols, toks[g], parts[g], part_len, &holders[g], &pending[g]);
         if (rc != LNH_OK) return rc;
         mats[g] = holders[g]->m;
         any = mats[g];
@@ -313,6 +340,8 @@ int lnq_gemm_grouped(uint32_t type, size_t n_cols, size_t n_rows, size_t n_group
         }
         commit(s, pending[g]);
     }
+    for (size_t g = 0; g < n_groups; g++)
+        if (holders[g]) recharge(s, holders[g]->m);
     return LNH_OK;
 }
 

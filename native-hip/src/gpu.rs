@@ -26,7 +26,7 @@ impl HipMatrix {
         self.shape
     }
 
-    /// Bytes this matrix holds in device memory (every layout it is kept in).
+    /// Bytes this matrix holds in device memory now (it grows once, when the multi-token layout is made).
     pub fn device_bytes(&self) -> usize {
         let mut bytes = 0usize;
         // SAFETY: `raw` is a live matrix handle; the three unused outputs may be null.
@@ -122,6 +122,14 @@ impl HipGemv {
     pub fn gemm_resident(&mut self, matrix: &HipMatrix, tokens: usize, input: &[f32], output: &mut [f32]) -> Result<(), String> {
         // SAFETY: as for gemv_resident.
         self.check(unsafe { ffi::lnh_gemm(self.raw, matrix.raw, tokens, input.as_ptr(), input.len(), output.as_mut_ptr(), output.len()) })
+    }
+
+    /// Makes now what products of up to `max_tokens` tokens by `matrix` need beyond the upload (the multi-token
+    /// layout of a quantized matrix is otherwise made by the first such product). For callers that run products
+    /// where nothing may be allocated, e.g. while a stream is being captured.
+    pub fn prepare(&mut self, matrix: &HipMatrix, max_tokens: usize) -> Result<(), String> {
+        // SAFETY: both handles are live and belong together (checked by the library).
+        self.check(unsafe { ffi::lnh_matrix_prepare(self.raw, matrix.raw, max_tokens) })
     }
 
     /// The per-expert products of one MoE projection in one call: group `g` multiplies `tokens[g]`

@@ -36,6 +36,7 @@ mod ffi {
         pub fn lnh_upload_packed_device(exec: *mut LnhExec, ggml_type: u32, rows: usize, cols: usize, device_bytes: *const c_void, nbytes: usize, out: *mut *mut LnhMatrix) -> c_int;
         pub fn lnh_matrix_free(matrix: *mut LnhMatrix);
         pub fn lnh_matrix_info(matrix: *const LnhMatrix, ggml_type: *mut u32, rows: *mut usize, cols: *mut usize, device_bytes: *mut usize) -> c_int;
+        pub fn lnh_matrix_prepare(exec: *mut LnhExec, matrix: *const LnhMatrix, max_tokens: usize) -> c_int;
         pub fn lnh_gemv(exec: *mut LnhExec, matrix: *const LnhMatrix, x: *const f32, x_len: usize, y: *mut f32, y_len: usize) -> c_int;
         pub fn lnh_gemm(exec: *mut LnhExec, matrix: *const LnhMatrix, tokens: usize, x: *const f32, x_len: usize, y: *mut f32, y_len: usize) -> c_int;
         pub fn lnh_gemv_once(exec: *mut LnhExec, weights: *const f32, weights_len: usize, x: *const f32, x_len: usize, y: *mut f32, y_len: usize) -> c_int;

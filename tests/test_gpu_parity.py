@@ -233,10 +233,10 @@ def test_invalid_operations_preserve_output_with_a_live_device(pkg):
 
 
 def test_workspace_growth_under_stream_capture_is_refused_not_recorded(pkg):
-    """A multi-token product whose workspace does not exist yet cannot be captured into a HIP graph (growing
-    allocates): the call fails with nothing launched and the capture stays usable.  The allocation-free entry
-    point can be captured at once, and the ordinary one after one eager call; replays of both equal the eager
-    result bit for bit."""
+    """A multi-token product that would have to allocate cannot be captured into a HIP graph: while the matrix has
+    no multi-token layout both entry points fail with nothing launched; once lnh_matrix_prepare has made it the
+    allocation-free entry point can be captured at once and the ordinary one after one eager call (its workspace
+    grows then); the capture stays usable throughout and replays of both equal the eager result bit for bit."""
     hip = importlib.import_module("llama-rust_amd.hiprt")
     g = pkg.HipGemv(0)  # a fresh executor: no workspace yet
     rng = np.random.default_rng(31)
@@ -248,6 +248,21 @@ def test_workspace_growth_under_stream_capture_is_refused_not_recorded(pkg):
     ya, yb, yc = (hip.DeviceBuffer(tokens * rows * 4) for _ in range(3))
     stream = hip.Stream()
     seen = {}
+    unprepared = []
+
+    def enqueue_unprepared(s):   # the matrix has only been uploaded: its multi-token layout does not exist yet
+        for call in (g.gemm_device, g.gemm_device_noalloc):
+            try:
+                call(m, tokens, xd.ptr, ya.ptr, s.ptr)
+            except pkg.NativeHipError as e:
+                unprepared.append((e.code, str(e)))
+
+    single = m.info()[3]
+    hip.Graph(stream, enqueue_unprepared).destroy()
+    assert [c for c, _ in unprepared] == [pkg.ERR_INVALID] * 2 and all("lnh_matrix_prepare" in t for _, t in unprepared)
+    assert m.info()[3] == single                 # nothing was made under the capture
+    g.prepare(m, tokens)
+    assert m.info()[3] > single
 
     def enqueue(s):
         try:
@@ -693,6 +708,56 @@ def test_residency_lru_and_budget(pkg, monkeypatch):
     pkg.reset()
     run(mats[0])
     assert pkg.cache_stats()["limit"] > (1 << 30)    # automatic budget on a 288 GB device
+
+
+def test_residency_charges_the_multi_token_layout_when_it_appears(pkg, monkeypatch):
+    """A cached matrix is charged for what it holds on the device: the single-token layout from its upload, the
+    multi-token layout from the first product of three or more tokens on (it is made then, not before).  A
+    budget that takes the first and not both keeps the matrix while it only meets single tokens and drops it
+    after the product that made it grow."""
+    rng = np.random.default_rng(21)
+    rows, cols = 256, 512
+    w = K.random_packed(K.Q4_K, rows, cols, rng, signed=False, scale=0.02)
+    g = pkg.HipGemv(0)
+    probe = g.upload_packed(K.Q4_K, rows, cols, w)
+    single = probe.info()[3]
+    g.prepare(probe, 8)
+    both = probe.info()[3]
+    probe.close()
+    g.close()
+    assert both > single
+
+    def run(tokens):
+        x = rng.normal(0, 1, tokens * cols).astype(np.float32)
+        y = np.full(tokens * rows, np.nan, np.float32)
+        pkg.gemm(K.Q4_K, cols, tokens, w, x, y)
+        check(y, K.Q4_K, cols, tokens, rows, w, x)
+
+    monkeypatch.setenv("LLAMA_HIP_CACHE_BYTES", str(1 << 30))
+    pkg.reset()
+    run(1)
+    assert pkg.cache_stats()["bytes"] == single + w.size
+    run(2)                                            # two tokens are two single-token launches
+    assert pkg.cache_stats()["bytes"] == single + w.size
+    run(8)
+    s = pkg.cache_stats()
+    assert s["bytes"] == both + w.size and s["entries"] == 1 and s["hits"] == 2
+    pkg.reset()
+    run(8)                                            # a miss that is a multi-token product is charged in full at once
+    assert pkg.cache_stats()["bytes"] == both + w.size
+
+    monkeypatch.setenv("LLAMA_HIP_CACHE_BYTES", str(single + w.size + 16))
+    pkg.reset()
+    run(1); run(1)
+    s = pkg.cache_stats()
+    assert s["entries"] == 1 and s["hits"] == 1
+    run(8)                                            # correct result, then over budget: not kept
+    s = pkg.cache_stats()
+    assert s["entries"] == 0 and s["bytes"] == 0
+    run(8)                                            # over budget from the start: runs once, never retained
+    assert pkg.cache_stats()["entries"] == 0
+    monkeypatch.delenv("LLAMA_HIP_CACHE_BYTES")
+    pkg.reset()
 
 
 def test_edge_sample_collision_does_not_alias(pkg):

@@ -63,6 +63,9 @@ def test_noalloc_equals_gemm_device_twice_in_a_row(gpu, hip, ty):
     w2 = K.random_packed(ty, rows2, cols2, rng, signed=False, scale=0.02)
     m2 = gpu.upload_packed(ty, rows2, cols2, w2)
     try:
+        # the entry point allocates nothing, so what the multi-token kernels read must exist before it is called
+        gpu.prepare(m, 40)
+        gpu.prepare(m2, 5)
         _both(gpu, hip, m, ty, rows, cols, 40, w, rng)
         _both(gpu, hip, m2, ty, rows2, cols2, 5, w2, rng)
         _both(gpu, hip, m, ty, rows, cols, 9, w, rng)
@@ -83,6 +86,15 @@ def test_noalloc_rejects_what_does_not_fit(gpu, hip, pkg):
     yd = hip.DeviceBuffer(tokens * rows * 4)
     yd.fill_byte(0x5a)
     try:
+        # a matrix that has only been uploaded has no multi-token layout yet, and this entry point may not make it
+        with pytest.raises(pkg.NativeHipError) as ei:
+            gpu.gemm_device_noalloc(m, 4, xd.ptr, yd.ptr)
+        assert ei.value.code == pkg.ERR_INVALID and "lnh_matrix_prepare" in str(ei.value)
+        single = m.info()[3]
+        gpu.prepare(m, 1)                       # a single token needs nothing more
+        assert m.info()[3] == single
+        gpu.prepare(m, 4)
+        assert m.info()[3] > single
         with pytest.raises(pkg.NativeHipError) as ei:
             gpu.gemm_device_noalloc(m, tokens, xd.ptr, yd.ptr)
         assert ei.value.code == pkg.ERR_INVALID and "allocation-free" in str(ei.value)
