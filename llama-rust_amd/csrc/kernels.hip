@@ -616,7 +616,67 @@ static hipError_t launch_mm(hipStream_t stream, MmPlan &p, void *ws, size_t ws_b
     }
 }
 
-// Single-token products, and F32/F16 products of any token count.
+// F32 / F16 weights, two or more tokens: gemm_fmfma_kernel (+ fg_reduce_kernel when columns are shared).
+struct FgPlan {
+    FgJob job;
+    int tt;
+    uint32_t wgs;
+    size_t part_bytes;
+};
+static void fg_plan(const MatView &m, uint32_t tokens, FgPlan &p) {
+    p.tt = tokens > 32 ? 2 : 1;
+    const uint32_t tile_tok = 32u * (uint32_t)p.tt;
+    const uint32_t tok_tiles = (tokens + tile_tok - 1) / tile_tok, row_tiles = (m.rows + FG_ROWS - 1) / FG_ROWS;
+    const uint32_t tiles = tok_tiles * row_tiles, n_steps = (m.cols + FG_K - 1) / FG_K;
+    uint32_t ks = (uint32_t)(2 * g_cu_count) / (tiles ? tiles : 1);   // about two workgroups per CU
+    if (ks > n_steps / 8) ks = n_steps / 8;                           // a share is at least 256 columns
+    if (ks > 32) ks = 32;
+    if (ks < 1) ks = 1;
+    p.job.m = m;
+    p.job.x = nullptr;
+    p.job.y = nullptr;
+    p.job.part = nullptr;
+    p.job.tokens = tokens;
+    p.job.tok_tiles = tok_tiles;
+    p.job.ksplit = ks;
+    p.job.pad = 0;
+    p.wgs = tiles * ks;
+    p.part_bytes = ks > 1 ? up256((size_t)ks * tokens * m.rows * sizeof(float)) : 0;
+}
+
+template <uint32_t T, int TT>
+static hipError_t launch_fg_main(hipStream_t stream, const FgPlan &p) {
+    constexpr size_t lds = (size_t)2 * (FG_ROWS + 32 * TT) * FG_LD * sizeof(float);
+    auto kern = gemm_fmfma_kernel<T, TT>;
+    static bool configured = false;
+    if (lds > 48 * 1024 && !configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(p.wgs), dim3(256), lds, stream, p.job);
+    return hipGetLastError();
+}
+
+static hipError_t launch_fg(hipStream_t stream, const MatView &m, uint32_t tokens, const float *x, float *y, void *ws,
+                            size_t ws_bytes) {
+    FgPlan p;
+    fg_plan(m, tokens, p);
+    if (p.part_bytes > ws_bytes) return hipErrorInvalidValue;
+    p.job.x = x;
+    p.job.y = y;
+    p.job.part = static_cast<float *>(ws);
+    hipError_t e;
+    if (m.type == T_F16) e = p.tt == 2 ? launch_fg_main<T_F16, 2>(stream, p) : launch_fg_main<T_F16, 1>(stream, p);
+    else e = p.tt == 2 ? launch_fg_main<T_F32, 2>(stream, p) : launch_fg_main<T_F32, 1>(stream, p);
+    if (e != hipSuccess || p.job.ksplit < 2) return e;
+    const size_t total = (size_t)tokens * m.rows, vec = (total + 3) / 4, blocks = (vec + 255) / 256;
+    hipLaunchKernelGGL(fg_reduce_kernel, dim3((unsigned)(blocks < 512 ? blocks : 512)), dim3(256), 0, stream, p.job.part, y, total,
+                       p.job.ksplit);
+    return hipGetLastError();
+}
+
+// Single-token products, and whatever the other paths do not take.
 static hipError_t launch_plain(hipStream_t stream, const MatView &m, uint32_t tokens, const float *x, float *y) {
     auto run = [&](auto tag) -> hipError_t {
         constexpr uint32_t T = decltype(tag)::value;
@@ -679,7 +739,15 @@ size_t gemm_workspace_bytes(const MatView *mats, const uint32_t *tokens, uint32_
     for (uint32_t g = 0; g < n;) {
         if (tokens[g] == 0 || mats[g].rows == 0) { g++; continue; }
         const uint32_t run = mm_run(mats, tokens, n, g);
-        if (run == 0) { g++; continue; }
+        if (run == 0) {
+            if ((mats[g].type == T_F32 || mats[g].type == T_F16) && tokens[g] > 1) {
+                FgPlan p;
+                fg_plan(mats[g], tokens[g], p);
+                need = p.part_bytes > need ? p.part_bytes : need;
+            }
+            g++;
+            continue;
+        }
         MmClass cls[2];
         mm_classes(mats + g, tokens + g, nullptr, nullptr, run, cls);
         for (const MmClass &c : cls) {
@@ -704,6 +772,8 @@ hipError_t launch_gemm_groups(hipStream_t stream, const MatView *mats, const Mat
             if (mm_type(mats[g].type) && tokens[g] > 1) {
                 for (uint32_t t = 0; t < tokens[g] && e == hipSuccess; t++)
                     e = launch_plain(stream, mats[g], 1, xs[g] + (size_t)t * mats[g].cols, ys[g] + (size_t)t * mats[g].rows);
+            } else if ((mats[g].type == T_F32 || mats[g].type == T_F16) && tokens[g] > 1) {
+                e = launch_fg(stream, mats[g], tokens[g], xs[g], ys[g], ws, ws_bytes);
             } else {
                 e = launch_plain(stream, mats[g], tokens[g], xs[g], ys[g]);
             }

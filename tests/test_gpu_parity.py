@@ -329,6 +329,30 @@ def test_a_failed_product_leaves_no_cache_entry_behind(pkg):
 
 
 # ------------------------------------------------------------------ random data, all dtypes
+@pytest.mark.parametrize("ty", [K.F16, K.F32], ids=lambda t: O.TYPE_NAMES[t])
+def test_plain_dtypes_on_the_matrix_cores_every_tile_and_share_shape(pkg, gpu, ty):
+    """F16 / F32 weights with two or more tokens run on the f32 matrix instruction: 128-row and 32- or 64-token
+    tiles, columns in steps of 32 shared between workgroups when rows and tokens alone leave CUs idle.  Shapes on
+    both sides of every tile edge, rows that are not whole 16-byte groups (activations then load element by
+    element), a single step, many shares, token counts across the 32 / 64 switch and beyond one tile."""
+    rng = np.random.default_rng(4000 + ty)
+    for rows, cols in ((127, 32), (128, 31), (129, 33), (1, 4096), (260, 1030), (96, 8192), (512, 14336), (31, 3)):
+        w = K.random_packed(ty, rows, cols, rng)
+        m = gpu.upload_packed(ty, rows, cols, w)
+        for tokens in (2, 3, 31, 32, 33, 64, 65, 130):
+            x = rng.normal(0, 1, tokens * cols).astype(np.float32)
+            y = np.full(tokens * rows, np.nan, np.float32)
+            gpu.gemm_resident(m, tokens, x, y)
+            check(y, ty, cols, tokens, rows, w, x, f"{O.TYPE_NAMES[ty]} {rows}x{cols} M={tokens}")
+            if tokens in (3, 65):   # row t of a batch is the product of token t alone, up to the order of the sums
+                t = tokens - 1
+                alone = np.full(rows, np.nan, np.float32)
+                gpu.gemm_resident(m, 1, x[t * cols:(t + 1) * cols], alone)
+                exact, mag = O.gemm_f64_mag(ty, cols, 1, w, x[t * cols:(t + 1) * cols], rows)
+                assert np.all(np.abs(y.reshape(tokens, rows)[t] - alone) <= 2 * K.single_kernel_bound(cols, mag))
+        m.close()
+
+
 @pytest.mark.parametrize("ty", O.ALL_TYPES, ids=lambda t: O.TYPE_NAMES[t])
 def test_random_gemv_and_gemm_within_bounds(pkg, gpu, ty):
     """Signed scales, every code value, int8 -128, token counts across the kernel switch points."""
