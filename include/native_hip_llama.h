@@ -95,6 +95,14 @@ void lnm_session_free(lnm_session *session);
 /* Runs the n tokens as one batch at positions past .. past+n-1 (products with n_tokens = n) and
  * writes the logits of the last one (n_vocab floats). */
 int lnm_forward(lnm_session *session, const uint32_t *tokens, size_t n, float *logits);
+/* A whole prompt for a session that may already hold part of it (the reference's prompt_logits with prefix
+ * reuse, langtax/src/decode.rs:1106-1196, 3931-3962; its test scenario langtax/tests/native_cuda_parity.rs:236-249):
+ * the session remembers the tokens it has forwarded; positions 0 .. lcp-1 of the cache are kept, where lcp is
+ * the longest common prefix of those tokens and `tokens`, the rest is forwarded as one batch at positions
+ * lcp .. n-1 and replaces what the cache held there.  A full hit (lcp == n) recomputes the last token, so the
+ * logits are always those of tokens[n-1].  `prefix_hit` (may be NULL) receives lcp.  A session whose remembered
+ * tokens do not cover its cache (after a failed call) starts over from position 0. */
+int lnm_prompt(lnm_session *session, const uint32_t *tokens, size_t n, float *logits, size_t *prefix_hit);
 /* Greedy decode: the prompt as one batch, then one token at a time; out[0] comes from the prompt's
  * logits, out[i] from decode step i, n_new tokens and n_new - 1 decode steps in all.  The two
  * wall times (seconds) may be NULL. */

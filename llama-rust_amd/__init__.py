@@ -138,6 +138,7 @@ def load_library():
         "lnm_batch_generate_greedy": (C.c_int, [vp, vp, vp, sz, vp, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
         "lnm_session_free": (None, [vp]),
         "lnm_forward": (C.c_int, [vp, vp, sz, vp]),
+        "lnm_prompt": (C.c_int, [vp, vp, sz, vp, vp]),
         "lnm_generate_greedy": (C.c_int, [vp, vp, sz, sz, vp, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
         "lnm_session_timing": (C.c_int, [vp, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_uint64)]),
         "lnm_dequant_row": (C.c_int, [u32, sz, vp, sz, vp]),

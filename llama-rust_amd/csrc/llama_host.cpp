@@ -383,6 +383,7 @@ struct lnm_session {
     lnm_model *model = nullptr;
     std::unique_ptr<DeviceDecode, void (*)(DeviceDecode *)> dev{nullptr, nullptr};  // set: the whole step runs on the GPU
     size_t kv_block = 16, past = 0;
+    std::vector<uint32_t> ids;        // the tokens at positions 0 .. past-1, for lnm_prompt's prefix reuse
     std::vector<uint32_t> table;      // logical block -> physical block
     std::vector<uint32_t> preset;     // physical ids to hand out, in order (empty: 0, 1, 2, ...)
     std::vector<float> cache_k, cache_v;
@@ -1084,8 +1085,25 @@ void lnm_session_free(lnm_session *session) { delete session; }
 int lnm_forward(lnm_session *session, const uint32_t *tokens, size_t n, float *logits) {
     if (!session || !tokens || !logits) return fail("null argument");
     if (session->dev && session->dev->n_seq) return fail("a batch session takes lnm_batch_generate_greedy");
-    if (session->dev) return device_forward(session, tokens, n, logits);
-    return forward(session, tokens, n, logits);
+    const int rc = session->dev ? device_forward(session, tokens, n, logits) : forward(session, tokens, n, logits);
+    if (rc == 0) session->ids.insert(session->ids.end(), tokens, tokens + n);
+    return rc;
+}
+
+// langtax/src/decode.rs:1106-1196 (reuse_prefix, rewind, prompt_suffix) and 3931-3962 (prompt_logits).
+int lnm_prompt(lnm_session *session, const uint32_t *tokens, size_t n, float *logits, size_t *prefix_hit) {
+    if (!session || !tokens || !logits) return fail("null argument");
+    if (n == 0) return fail("prefill tokens");
+    if (session->dev && session->dev->n_seq) return fail("a batch session takes lnm_batch_generate_greedy");
+    size_t lcp = 0;
+    if (session->ids.size() == session->past)  // ids that do not cover the cache are no basis for reuse
+        while (lcp < session->ids.size() && lcp < n && session->ids[lcp] == tokens[lcp]) lcp++;
+    if (prefix_hit) *prefix_hit = lcp;
+    if (lcp == n) lcp = n - 1;  // a full hit recomputes the last token: the logits returned are that token's
+    // positions 0 .. lcp-1 stay as they are; everything after them is written again as the sequence grows
+    session->past = lcp;
+    session->ids.resize(lcp);
+    return lnm_forward(session, tokens + lcp, n - lcp, logits);
 }
 
 int lnm_generate_greedy(lnm_session *session, const uint32_t *prompt, size_t n_prompt, size_t n_new,
@@ -1093,7 +1111,22 @@ int lnm_generate_greedy(lnm_session *session, const uint32_t *prompt, size_t n_p
     if (!session || !prompt || !out) return fail("null argument");
     if (n_prompt == 0 || n_new == 0) return fail("empty prompt or nothing to generate");
     if (session->dev && session->dev->n_seq) return fail("a batch session takes lnm_batch_generate_greedy");
-    if (session->dev) return device_generate(session, prompt, n_prompt, n_new, out, prefill_seconds, decode_seconds);
+    struct Remember {  // on success the cache holds the prompt and every picked token but the last
+        lnm_session *s; const uint32_t *prompt; size_t n_prompt, n_new; const uint32_t *out; size_t past0; bool ok = false;
+        ~Remember() {
+            if (!ok || s->past != past0 + n_prompt + n_new - 1) {
+                s->ids.clear();
+                return;
+            }
+            s->ids.insert(s->ids.end(), prompt, prompt + n_prompt);
+            s->ids.insert(s->ids.end(), out, out + n_new - 1);
+        }
+    } remember{session, prompt, n_prompt, n_new, out, session->past};
+    if (session->dev) {
+        const int rc = device_generate(session, prompt, n_prompt, n_new, out, prefill_seconds, decode_seconds);
+        remember.ok = rc == 0;
+        return rc;
+    }
     std::vector<float> logits(session->model->hp.n_vocab);
     using clock = std::chrono::steady_clock;
     const auto t0 = clock::now();
@@ -1107,6 +1140,7 @@ int lnm_generate_greedy(lnm_session *session, const uint32_t *prompt, size_t n_p
     const auto t2 = clock::now();
     if (prefill_seconds) *prefill_seconds = std::chrono::duration<double>(t1 - t0).count();
     if (decode_seconds) *decode_seconds = std::chrono::duration<double>(t2 - t1).count();
+    remember.ok = true;
     return 0;
 }
 

@@ -239,6 +239,16 @@ class Session:
         _check(_pkg.load_library().lnm_forward(self._h, t.ctypes.data, t.size, logits.ctypes.data))
         return logits
 
+    def prompt(self, tokens):
+        """(logits of the last of `tokens`, reused prefix length): `tokens` as the whole sequence, keeping the
+        cached positions of the longest prefix it shares with what the session has forwarded so far
+        (langtax/src/decode.rs:3956-3962)."""
+        t = np.ascontiguousarray(tokens, dtype=np.uint32)
+        logits = np.empty(self.model.hparams.n_vocab, dtype=np.float32)
+        hit = C.c_size_t()
+        _check(_pkg.load_library().lnm_prompt(self._h, t.ctypes.data, t.size, logits.ctypes.data, C.byref(hit)))
+        return logits, hit.value
+
     def generate_greedy(self, prompt, n_new):
         """(tokens, prefill seconds, decode seconds): n_new tokens, the first from the prompt's logits."""
         p = np.ascontiguousarray(prompt, dtype=np.uint32)

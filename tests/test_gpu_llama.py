@@ -131,6 +131,47 @@ def test_small_model_with_experts_generates_the_same_tokens_as_the_cpu_path(pkg,
     assert len(set(toks_c)) >= 15  # the layers matter: no fixed point, no short cycle
 
 
+@pytest.mark.parametrize("kind", ["f32", "q4_0", "q4_k", "experts"])
+def test_reference_session_scenario_on_every_path(pkg, llama, tmp_path, kind):
+    """langtax/tests/native_cuda_parity.rs:198-249 for its four tiny models (F32, Q4_0, Q4_K weights, a model
+    with experts): prefill [1, 2, 3], decode 4, 5, 1, then the divergent full prompt [1, 2, 4], which keeps the
+    cached prefix [1, 2] and replaces the rest; a session with blocks of 2 positions beside one with large blocks.
+    Here on three paths: host session over the HIP products, device session, host session over the CPU oracle."""
+    spec = dict(n_layer=2, n_embd=256, n_head=4, n_head_kv=2, n_ff=512, n_vocab=96, seed=5, weight_std=0.06)
+    if kind == "f32":
+        spec.update(block_type=0, embd_type=0, output_type=0)
+    elif kind == "q4_0":
+        spec.update(block_type=2, embd_type=2, output_type=2)
+    elif kind == "q4_k":
+        spec.update(block_type=12, embd_type=12, output_type=14)
+    else:
+        spec.update(block_type=8, embd_type=8, output_type=8, n_expert=4, n_expert_used=2)
+    path = tmp_path / "tiny.gguf"
+    llama.write_synthetic_llama(path, **spec)
+    gpu = llama.Llama(path=path)
+    cpu = llama.Llama(path=path, products=llama.CALLBACK, matmul=cpu_products(False, 1))
+    snapshots = {}
+    for name, make in [("cpu", lambda kb: cpu.session(kv_block=kb)), ("host", lambda kb: gpu.session(kv_block=kb)),
+                       ("device", lambda kb: gpu.session(kv_block=kb, device_positions=32))]:
+        if name == "device" and kind == "experts":
+            continue  # the device session is for dense models (it refuses others, tested elsewhere)
+        for kb in (32, 2):
+            s = make(kb)
+            got = [s.forward([1, 2, 3])]
+            got += [s.forward([t]) for t in (4, 5, 1)]
+            reused, hit = s.prompt([1, 2, 4])
+            assert hit == 2
+            got.append(reused)
+            fresh = make(kb).forward([1, 2, 4])
+            assert np.abs(reused - fresh).max() <= 1e-5 * np.abs(fresh).max(), (name, kb)
+            snapshots[(name, kb)] = np.stack(got)
+    want = snapshots[("cpu", 32)]
+    scale = np.abs(want).max()
+    for key, got in snapshots.items():
+        assert np.abs(got - want).max() <= 1e-4 * scale, key
+        assert got.argmax(axis=1).tolist() == want.argmax(axis=1).tolist(), key
+
+
 def test_mixtral_shaped_routed_layer_matches_the_cpu_path(pkg, llama, tmp_path):
     """Benchmark configuration 5 as one checked result: 64 tokens, router logits of about unit deviation,
     softmax, top-2 of 8 experts, tokens grouped per expert, Q4_K gate / up (4096 -> 14336) and down

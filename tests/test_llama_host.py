@@ -313,6 +313,42 @@ def test_greedy_generation_is_prefill_then_single_token_steps(llama, tiny_path):
         m.session().generate_greedy([], 3)
 
 
+def test_prompt_reuses_the_cached_prefix_and_replaces_the_rest(llama, tiny_path):
+    """The reference's session scenario (langtax/tests/native_cuda_parity.rs:208-249): prefill [1, 2, 3], decode
+    4, 5, 1, then the divergent full prompt [1, 2, 4]; reuse rule of langtax/src/decode.rs:1106-1196."""
+    m = llama.Llama(path=tiny_path, products=llama.CALLBACK, matmul=oracle_matmul)
+    bits = lambda a: a.view(np.uint32).tolist()
+    for kv_block in (16, 2):  # its dense and its paged session (blocks of 2)
+        s = m.session(kv_block=kv_block)
+        s.forward([1, 2, 3])
+        for t in (4, 5, 1):
+            s.forward([t])
+        got, hit = s.prompt([1, 2, 4])
+        assert hit == 2
+        want = m.session(kv_block=kv_block).forward([1, 2, 4])
+        assert bits(got) == bits(want)
+        # the replaced positions really hold the new sequence: going on from it equals going on from scratch
+        fresh = m.session(kv_block=kv_block)
+        fresh.forward([1, 2, 4])
+        assert bits(s.forward([7])) == bits(fresh.forward([7]))
+        # a full hit recomputes the last token and reports the whole length
+        again, hit = s.prompt([1, 2, 4, 7])
+        assert hit == 4 and bits(again) == bits(m.session(kv_block=kv_block).forward([1, 2, 4, 7]))
+        # a longer prompt continues after the cached part; no common prefix starts over
+        longer, hit = s.prompt([1, 2, 4, 7, 30, 31])
+        assert hit == 4 and bits(longer) == bits(m.session(kv_block=kv_block).forward([1, 2, 4, 7, 30, 31]))
+        other, hit = s.prompt([9, 2, 4])
+        assert hit == 0 and bits(other) == bits(m.session(kv_block=kv_block).forward([9, 2, 4]))
+    # greedy generation leaves the prompt and all picked tokens but the last in the cache
+    s = m.session()
+    out, _, _ = s.generate_greedy([5, 1, 44], 4)
+    seq = [5, 1, 44] + out[:3].tolist()
+    _, hit = s.prompt(seq + [int(out[3])])
+    assert hit == len(seq)
+    with pytest.raises(llama.LlamaError, match="prefill tokens"):
+        s.prompt([])
+
+
 def test_synthetic_weights_have_the_requested_spread_for_every_dtype(llama, pkg, tmp_path):
     """Mean 0 and the requested standard deviation (within sampling noise) for all eight dtypes, and
     the generator is deterministic in its seed."""
