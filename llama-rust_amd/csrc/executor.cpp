@@ -178,8 +178,10 @@ int ensure_workspace(lnh_exec *e, hipStream_t s, size_t bytes) {
 // The tiled copy of m, made now if no product has needed it yet.  Making it allocates, which a stream under capture
 // cannot record, and the copy must be complete before any stream reads it: the one-time build is followed by a
 // synchronisation of the building stream.
-int ensure_tiled(lnh_exec *e, hipStream_t s, const lnh_matrix *m) {
+// `view` (may be null) receives the copy's addresses, read under the matrix's lock.
+int ensure_tiled(lnh_exec *e, hipStream_t s, const lnh_matrix *m, nh::MatView *view = nullptr) {
     std::lock_guard<std::mutex> lock(m->lazy);
+    if (view) *view = m->tiled;
     if (m->tiled.p0) return LNH_OK;
     const nh::TiledSpec ts = nh::tiled_spec(m->view.type, m->view.rows, m->view.cols);
     if (ts.total == 0) return LNH_OK;
@@ -217,6 +219,7 @@ int ensure_tiled(lnh_exec *e, hipStream_t s, const lnh_matrix *m) {
     m->dev_tiled = dev;
     m->tiled_bytes = ts.total;
     m->tiled = t;
+    if (view) *view = t;
     return LNH_OK;
 }
 
@@ -228,11 +231,11 @@ int launch_products(lnh_exec *e, hipStream_t s, size_t n, const lnh_matrix *cons
     for (size_t g = 0; g < n; g++) {
         views[g] = mats[g]->view;
         toks[g] = (uint32_t)tokens[g];
+        tiled[g] = nh::MatView{};  // single-token products never look at it
         if (nh::product_reads_tiled(views[g].type, toks[g]) && views[g].rows != 0) {
-            const int rt = ensure_tiled(e, s, mats[g]);
+            const int rt = ensure_tiled(e, s, mats[g], &tiled[g]);
             if (rt != LNH_OK) return rt;
         }
-        tiled[g] = mats[g]->tiled;
     }
     int rc = ensure_workspace(e, s, nh::gemm_workspace_bytes(views.data(), toks.data(), (uint32_t)n));
     if (rc != LNH_OK) return rc;
@@ -616,13 +619,15 @@ int lnh_gemm_device_noalloc(lnh_exec *e, const lnh_matrix *m, size_t tokens, con
                     "product needs " + std::to_string(need) + " bytes of workspace, the allocation-free entry point holds " +
                         std::to_string(nh::STATIC_SCRATCH_BYTES) + ": use lnh_gemm_device or fewer tokens per call");
     hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
+    nh::MatView tiled{};
     if (nh::product_reads_tiled(m->view.type, tok32)) {
         std::lock_guard<std::mutex> lock(m->lazy);
         if (!m->tiled.p0)
             return fail(e, LNH_ERR_INVALID,
                         "the matrix has no multi-token copy yet and this entry point does not allocate: call lnh_matrix_prepare first");
+        tiled = m->tiled;
     }
-    const hipError_t h = nh::launch_gemm_groups(s, &m->view, &m->tiled, &tok32, &dx, &dy, 1, ws, nh::STATIC_SCRATCH_BYTES);
+    const hipError_t h = nh::launch_gemm_groups(s, &m->view, &tiled, &tok32, &dx, &dy, 1, ws, nh::STATIC_SCRATCH_BYTES);
     if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
     return LNH_OK;
 }
