@@ -195,6 +195,35 @@ int lnh_gemv_fused_device(lnh_exec *exec, size_t n_mats, const lnh_matrix *const
  * 67 M weights per matrix on this part): the caller then uses lnh_gemv_fused_device. */
 int lnh_gemv_swiglu_device(lnh_exec *exec, const lnh_matrix *gate, const lnh_matrix *up, const float *device_x,
                            float *device_h, int prologue, const float *device_x2, float eps, void *stream);
+/* Activations kept in the form the multi-token kernels read, for steps that stay on the device.  No counterpart in
+ * the reference, whose every product takes and returns plain f32 rows on the host (langtax/src/native_gpu.rs:124-213).
+ * A multi-token product is three launches: the activations are cut into three bf16 parts in the matrix's column
+ * order, the matrix-core launch writes one partial result per share of the columns, a third launch sums the shares.
+ * Between two products of a decode step lies only element-wise work; lnh_gemm_act_device does that work in the
+ * launch that sums the shares and leaves its result already cut for the next matrix, so a chain of products costs
+ * two launches each instead of three plus the element-wise kernels.
+ *   lnh_act_create        a buffer for up to max_tokens tokens of `cols` columns under matrices of `ggml_type`
+ *                         (LNH_ERR_UNSUPPORTED for F32 / F16, whose products take plain rows)
+ *   lnh_act_split_device  fills it from `tokens` plain f32 rows on the device
+ *   lnh_gemm_act_device   multiplies it by up to 8 resident matrices of that dtype and column count (tokens >= 3;
+ *                         LNH_ERR_UNSUPPORTED below: single-token launches take plain rows), then
+ *     LNH_EPILOGUE_NONE         device_ys[i] = mats[i] x                        (any number of matrices)
+ *     LNH_EPILOGUE_ADD_RMSNORM  device_residual += mats[0] x, then RMSNorm of the new residual times device_norm_w
+ *                               (langtax/src/decode.rs:2957 / 3043 and 11498-11513) into device_xn (plain rows, may
+ *                               be NULL) and into `next` (may be NULL), whose columns are the matrix's rows
+ *     LNH_EPILOGUE_SWIGLU       SiLU(mats[0] x) * (mats[1] x) (decode.rs:11826-11830, 2981-2984) into `next`
+ *   Sums run in share order and the row operations in the order of a one-workgroup-per-row kernel, so results
+ *   equal those of the three-launch product followed by separate element-wise kernels bit for bit.
+ * Like lnh_gemm_device it may grow the executor's workspace and make a matrix's multi-token layout on first use;
+ * neither is possible while the stream is being captured (run the step once before capturing it). */
+typedef struct lnh_act lnh_act;
+enum { LNH_EPILOGUE_NONE = 0, LNH_EPILOGUE_ADD_RMSNORM = 1, LNH_EPILOGUE_SWIGLU = 2 };
+int lnh_act_create(lnh_exec *exec, uint32_t ggml_type, size_t cols, size_t max_tokens, lnh_act **out);
+void lnh_act_free(lnh_act *act);
+int lnh_act_split_device(lnh_exec *exec, lnh_act *act, size_t tokens, const float *device_x, void *stream);
+int lnh_gemm_act_device(lnh_exec *exec, size_t n_mats, const lnh_matrix *const *mats, const lnh_act *x, size_t tokens,
+                        float *const *device_ys, int epilogue, float *device_residual, const float *device_norm_w, float eps,
+                        float *device_xn, lnh_act *next, void *stream);
 /* Measurement aid, no counterpart in the reference: a plain device-to-device copy kernel
  * (nbytes a multiple of 16) whose known traffic calibrates HBM byte counters. */
 int lnh_calibration_copy(lnh_exec *exec, void *device_dst, const void *device_src, size_t nbytes, void *stream);

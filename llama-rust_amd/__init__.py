@@ -37,6 +37,7 @@ TYPE_NAMES = {F32: "f32", F16: "f16", Q4_0: "q4_0", Q5_0: "q5_0", Q5_1: "q5_1", 
 
 OK, ERR_INVALID, ERR_DEVICE, ERR_OOM, ERR_FOREIGN, ERR_UNSUPPORTED = range(6)
 PROLOGUE_NONE, PROLOGUE_RMSNORM, PROLOGUE_SWIGLU = 0, 1, 2
+EPILOGUE_NONE, EPILOGUE_ADD_RMSNORM, EPILOGUE_SWIGLU = 0, 1, 2
 
 
 class NativeHipError(RuntimeError):
@@ -137,6 +138,10 @@ def load_library():
         "lnm_session_new_device_batch": (C.c_int, [vp, sz, sz, sz, pvp]),
         "lnm_batch_generate_greedy": (C.c_int, [vp, vp, vp, sz, vp, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
         "lnm_session_free": (None, [vp]),
+        "lnh_act_create": (C.c_int, [vp, C.c_uint32, sz, sz, vp]),
+        "lnh_act_free": (None, [vp]),
+        "lnh_act_split_device": (C.c_int, [vp, vp, sz, vp, vp]),
+        "lnh_gemm_act_device": (C.c_int, [vp, sz, vp, vp, sz, vp, C.c_int, vp, vp, C.c_float, vp, vp, vp]),
         "lnm_forward": (C.c_int, [vp, vp, sz, vp]),
         "lnm_prompt": (C.c_int, [vp, vp, sz, vp, vp]),
         "lnm_generate_greedy": (C.c_int, [vp, vp, sz, sz, vp, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
@@ -227,6 +232,24 @@ class HipMatrix:
     def close(self):
         if self._h:
             load_library().lnh_matrix_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Act:
+    """Split activations on the device (lnh_act)."""
+
+    def __init__(self, lib, handle):
+        self._lib, self._h = lib, handle
+
+    def close(self):
+        if getattr(self, "_h", None):
+            self._lib.lnh_act_free(self._h)
             self._h = None
 
     def __del__(self):
@@ -330,6 +353,26 @@ class HipGemv:
         """gemm_device with the library's fixed device workspace: never allocates (include/native_hip.h)."""
         self._check(self._lib.lnh_gemm_device_noalloc(self._h, matrix._h, tokens, C.c_void_p(x_ptr), C.c_void_p(y_ptr),
                                                       C.c_void_p(stream)))
+
+    def act_create(self, ggml_type, cols, max_tokens):
+        """A device buffer for activations in the form the multi-token kernels read (include/native_hip.h)."""
+        h = C.c_void_p()
+        self._check(self._lib.lnh_act_create(self._h, ggml_type, cols, max_tokens, C.byref(h)))
+        return Act(self._lib, h)
+
+    def act_split_device(self, act, tokens, x_ptr, stream=0):
+        self._check(self._lib.lnh_act_split_device(self._h, act._h, tokens, C.c_void_p(x_ptr), C.c_void_p(stream)))
+
+    def gemm_act_device(self, matrices, act, tokens, y_ptrs=None, epilogue=EPILOGUE_NONE, residual_ptr=0, norm_w_ptr=0,
+                        eps=0.0, xn_ptr=0, next_act=None, stream=0):
+        """Products of split activations; with an epilogue the step after the product runs where its shares are summed
+        and leaves its result split in next_act."""
+        n = len(matrices)
+        mats = (C.c_void_p * n)(*[m._h for m in matrices])
+        ys = (C.c_void_p * n)(*y_ptrs) if y_ptrs is not None else None
+        self._check(self._lib.lnh_gemm_act_device(self._h, n, mats, act._h, tokens, ys, epilogue, C.c_void_p(residual_ptr),
+                                                  C.c_void_p(norm_w_ptr), eps, C.c_void_p(xn_ptr),
+                                                  next_act._h if next_act is not None else None, C.c_void_p(stream)))
 
     def gemm_grouped_device(self, matrices, tokens, x_ptr, y_ptr, stream=0):
         n = len(matrices)

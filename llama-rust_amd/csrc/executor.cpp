@@ -44,6 +44,13 @@ struct lnh_matrix {
     mutable nh::MatView tiled{};
 };
 
+struct lnh_act {
+    std::shared_ptr<Ctx> ctx;
+    void *dev = nullptr;
+    size_t bytes = 0;
+    uint32_t type = 0, cols = 0, max_tokens = 0;
+};
+
 struct lnh_exec {
     std::shared_ptr<Ctx> ctx;
     hipStream_t stream = nullptr;
@@ -628,6 +635,127 @@ int lnh_gemm_device_noalloc(lnh_exec *e, const lnh_matrix *m, size_t tokens, con
         tiled = m->tiled;
     }
     const hipError_t h = nh::launch_gemm_groups(s, &m->view, &tiled, &tok32, &dx, &dy, 1, ws, nh::STATIC_SCRATCH_BYTES);
+    if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
+    return LNH_OK;
+}
+
+int lnh_act_create(lnh_exec *e, uint32_t type, size_t cols, size_t max_tokens, lnh_act **out) {
+    if (!e) return LNH_ERR_INVALID;
+    if (!out) return fail(e, LNH_ERR_INVALID, "output pointer is null");
+    *out = nullptr;
+    if (cols > UINT32_MAX || max_tokens > UINT32_MAX) return fail(e, LNH_ERR_INVALID, "activation shape exceeds u32");
+    const size_t bytes = nh::act_bytes(type, (uint32_t)cols, (uint32_t)max_tokens);
+    if (bytes == 0)
+        return fail(e, LNH_ERR_UNSUPPORTED, "split activations exist for the block-quantized dtypes, columns in multiples of 32 and at least one token");
+    hipError_t h = hipSetDevice(e->ctx->device);
+    if (h != hipSuccess) return hip_fail(e, h, "hipSetDevice");
+    void *dev = nullptr;
+    h = hipMalloc(&dev, bytes);
+    if (h != hipSuccess) return hip_fail(e, h, "HIP activation allocation");
+    // slots past the tokens of a call are multiplied like any other and dropped: keep them finite from the start
+    h = hipMemsetAsync(dev, 0, bytes, e->stream);
+    const hipError_t hs = hipStreamSynchronize(e->stream);
+    if (h == hipSuccess) h = hs;
+    if (h != hipSuccess) {
+        (void)hipFree(dev);
+        return hip_fail(e, h, "HIP activation allocation");
+    }
+    auto a = std::make_unique<lnh_act>();
+    a->ctx = e->ctx;
+    a->dev = dev;
+    a->bytes = bytes;
+    a->type = type;
+    a->cols = (uint32_t)cols;
+    a->max_tokens = (uint32_t)max_tokens;
+    *out = a.release();
+    return LNH_OK;
+}
+
+void lnh_act_free(lnh_act *a) {
+    if (!a) return;
+    if (a->dev) {
+        (void)hipSetDevice(a->ctx->device);
+        (void)hipFree(a->dev);
+    }
+    delete a;
+}
+
+int lnh_act_split_device(lnh_exec *e, lnh_act *a, size_t tokens, const float *dx, void *stream) {
+    if (!e) return LNH_ERR_INVALID;
+    if (!a || !dx) return fail(e, LNH_ERR_INVALID, "activation or buffer pointer is null");
+    if (a->ctx.get() != e->ctx.get()) return fail(e, LNH_ERR_FOREIGN, "activations belong to a different executor");
+    if (tokens == 0 || tokens > a->max_tokens) return fail(e, LNH_ERR_INVALID, "token count outside the activations' capacity");
+    hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
+    const hipError_t h = nh::launch_act_split(s, a->dev, a->type, a->cols, a->max_tokens, (uint32_t)tokens, dx);
+    if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
+    return LNH_OK;
+}
+
+int lnh_gemm_act_device(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, const lnh_act *x, size_t tokens,
+                        float *const *dys, int epilogue, float *d_residual, const float *d_norm_w, float eps, float *d_xn,
+                        lnh_act *next, void *stream) {
+    if (!e) return LNH_ERR_INVALID;
+    if (!mats || !x || n_mats == 0) return fail(e, LNH_ERR_INVALID, "matrix list or activations are null");
+    if (n_mats > 8) return fail(e, LNH_ERR_INVALID, "at most 8 matrices per call");
+    if (x->ctx.get() != e->ctx.get() || (next && next->ctx.get() != e->ctx.get()))
+        return fail(e, LNH_ERR_FOREIGN, "activations belong to a different executor");
+    if (tokens == 0 || tokens > x->max_tokens || (next && tokens > next->max_tokens))
+        return fail(e, LNH_ERR_INVALID, "token count outside the activations' capacity");
+    if (tokens < nh::MM_MIN_TOKENS)
+        return fail(e, LNH_ERR_UNSUPPORTED, "split activations serve products of three or more tokens");
+    nh::MatView views[8], tiled[8];
+    for (size_t i = 0; i < n_mats; i++) {
+        const lnh_matrix *m = mats[i];
+        if (!m) return fail(e, LNH_ERR_INVALID, "HIP matrix is null");
+        if (m->ctx.get() != e->ctx.get()) return fail(e, LNH_ERR_FOREIGN, "HIP matrix belongs to a different executor");
+        if (m->view.type != x->type || m->view.cols != x->cols)
+            return fail(e, LNH_ERR_INVALID, "the activations were split for another dtype or column count than the matrix has");
+        if (m->view.rows == 0) return fail(e, LNH_ERR_INVALID, "HIP matrix has no rows");
+        views[i] = m->view;
+    }
+    nh::ActEpilogue ep;
+    switch (epilogue) {
+    case LNH_EPILOGUE_NONE:
+        if (!dys) return fail(e, LNH_ERR_INVALID, "output list is null");
+        for (size_t i = 0; i < n_mats; i++)
+            if (!dys[i]) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+        break;
+    case LNH_EPILOGUE_ADD_RMSNORM:
+        if (n_mats != 1) return fail(e, LNH_ERR_INVALID, "the residual epilogue takes one matrix");
+        if (!d_residual || !d_norm_w) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+        if (next && next->cols != views[0].rows) return fail(e, LNH_ERR_INVALID, "next activations do not have the product's width");
+        ep.kind = nh::ACT_EPILOGUE_ADD_RMSNORM;
+        break;
+    case LNH_EPILOGUE_SWIGLU:
+        if (n_mats != 2 || views[0].rows != views[1].rows) return fail(e, LNH_ERR_INVALID, "SiLU(gate) * up takes two matrices of one shape");
+        if (!next) return fail(e, LNH_ERR_INVALID, "SiLU(gate) * up needs activations to leave its result in");
+        if (next->cols != views[0].rows) return fail(e, LNH_ERR_INVALID, "next activations do not have the product's width");
+        ep.kind = nh::ACT_EPILOGUE_SWIGLU;
+        break;
+    default: return fail(e, LNH_ERR_INVALID, "unknown epilogue");
+    }
+    ep.residual = d_residual;
+    ep.norm_w = d_norm_w;
+    ep.eps = eps;
+    ep.xn_out = d_xn;
+    if (next) {
+        ep.next_act = next->dev;
+        ep.next_type = next->type;
+        ep.next_cols = next->cols;
+        ep.next_max_tokens = next->max_tokens;
+    }
+    hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
+    for (size_t i = 0; i < n_mats; i++) {
+        const int rt = ensure_tiled(e, s, mats[i], &tiled[i]);
+        if (rt != LNH_OK) return rt;
+    }
+    int rc = ensure_workspace(e, s, nh::gemm_act_workspace_bytes(tiled, (uint32_t)n_mats, (uint32_t)tokens, ep.kind != nh::ACT_EPILOGUE_NONE));
+    if (rc != LNH_OK) return rc;
+    const hipError_t h = nh::launch_gemm_act(s, tiled, (uint32_t)n_mats, (uint32_t)tokens, x->dev, x->max_tokens, dys, ep, e->d_ws, e->ws_cap);
+    if (h == hipErrorInvalidValue) {
+        (void)hipGetLastError();
+        return fail(e, LNH_ERR_UNSUPPORTED, "this product is not one the split-activation path launches");
+    }
     if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
     return LNH_OK;
 }

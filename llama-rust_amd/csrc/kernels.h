@@ -37,6 +37,35 @@ hipError_t launch_gemm(hipStream_t stream, const MatView &m, const MatView &tile
 hipError_t launch_gemm_groups(hipStream_t stream, const MatView *mats, const MatView *tiled, const uint32_t *tokens,
                               const float *const *xs, float *const *ys, uint32_t n, void *ws, size_t ws_bytes);
 
+// Activations that stay in the form the matrix-core kernels read (three bf16 parts per group of 16 columns, in the
+// column order of the dtype that will multiply them) between products, for callers whose steps stay on the device:
+// act_bytes sizes a buffer for up to max_tokens tokens of `cols` columns under a matrix of dtype `type` (0: not a
+// dtype / shape of the matrix-core path); launch_act_split fills it from plain f32 rows; launch_gemm_act multiplies
+// it by n matrices of that dtype and column count (tiled copies, tokens >= 3) and either writes ys (epilogue NONE:
+// main launch + share sum, as launch_gemm_groups without its split launch) or applies, in the launch that sums the
+// shares, the step that follows the product and leaves the result split in next_act for the next product:
+//   ADD_RMSNORM (n = 1)   residual[t] += W x[t]; xn = RMSNorm(residual[t]) * norm_w -> xn_out (may be null), next_act
+//                         (may be null; next_cols = rows of W)
+//   SWIGLU (n = 2)        SiLU(W0 x[t]) * (W1 x[t]) -> next_act (next_cols = rows of W0 = rows of W1)
+// ws must hold gemm_act_workspace_bytes() for the same arguments.  hipErrorInvalidValue = not this path's case,
+// nothing launched.
+enum { ACT_EPILOGUE_NONE = 0, ACT_EPILOGUE_ADD_RMSNORM = 1, ACT_EPILOGUE_SWIGLU = 2 };
+struct ActEpilogue {
+    int kind = ACT_EPILOGUE_NONE;
+    float *residual = nullptr;
+    const float *norm_w = nullptr;
+    float eps = 0.f;
+    float *xn_out = nullptr;
+    void *next_act = nullptr;
+    uint32_t next_type = 0, next_cols = 0, next_max_tokens = 0;
+};
+size_t act_bytes(uint32_t type, uint32_t cols, uint32_t max_tokens);
+hipError_t launch_act_split(hipStream_t stream, void *act, uint32_t type, uint32_t cols, uint32_t max_tokens, uint32_t tokens,
+                            const float *x);
+size_t gemm_act_workspace_bytes(const MatView *mats, uint32_t n, uint32_t tokens, bool with_epilogue);
+hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n, uint32_t tokens, void *act, uint32_t act_max_tokens,
+                           float *const *ys, const ActEpilogue &ep, void *ws, size_t ws_bytes);
+
 // One launch for up to 8 single-token products that read the same x and share dtype
 // and column count (q/k/v, gate/up).  hipErrorInvalidValue = not fusable this way;
 // the caller then launches them one by one.  accumulate: y += W x instead of y = W x.

@@ -794,6 +794,171 @@ hipError_t launch_gemm_groups(hipStream_t stream, const MatView *mats, const Mat
     return hipSuccess;
 }
 
+// ---- activations that stay in the split form between products
+
+static uint32_t act_mpad(uint32_t type, uint32_t tokens) { return tokens + (tokens <= 16 && type != T_Q6_K ? 16u : 64u); }
+
+size_t act_bytes(uint32_t type, uint32_t cols, uint32_t max_tokens) {
+    if (!mm_type(type) || cols % 32 != 0 || max_tokens == 0) return 0;
+    const size_t n_groups = cols / 16, mpad = (size_t)max_tokens + 64;
+    return up256(n_groups * 6 * mpad * sizeof(uint4)) + up256(n_groups * mpad * sizeof(float));
+}
+
+// Where `tokens` tokens lie in an activation buffer made for up to max_tokens (the slot stride follows the token
+// count, as in a product's own workspace; the sums start where the planes of max_tokens would end).
+static ActView act_view(void *act, uint32_t type, uint32_t cols, uint32_t max_tokens, uint32_t tokens) {
+    ActView v;
+    const size_t n_groups = cols / 16;
+    v.xb = static_cast<uint4 *>(act);
+    v.sx = reinterpret_cast<float *>(static_cast<uint8_t *>(act) + up256(n_groups * 6 * ((size_t)max_tokens + 64) * sizeof(uint4)));
+    v.mpad = act_mpad(type, tokens);
+    v.n_groups = (uint32_t)n_groups;
+    return v;
+}
+
+template <typename F> static hipError_t mm_by_type(uint32_t type, F &&run) {
+    switch (type) {
+    case T_Q4_0: return run(std::integral_constant<uint32_t, T_Q4_0>{});
+    case T_Q5_0: return run(std::integral_constant<uint32_t, T_Q5_0>{});
+    case T_Q5_1: return run(std::integral_constant<uint32_t, T_Q5_1>{});
+    case T_Q8_0: return run(std::integral_constant<uint32_t, T_Q8_0>{});
+    case T_Q4_K: return run(std::integral_constant<uint32_t, T_Q4_K>{});
+    case T_Q6_K: return run(std::integral_constant<uint32_t, T_Q6_K>{});
+    default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_act_split(hipStream_t stream, void *act, uint32_t type, uint32_t cols, uint32_t max_tokens, uint32_t tokens,
+                            const float *x) {
+    if (!act || !x || act_bytes(type, cols, max_tokens) == 0 || tokens == 0 || tokens > max_tokens) return hipErrorInvalidValue;
+    const ActView v = act_view(act, type, cols, max_tokens, tokens);
+    MmBatch b{};
+    b.job[0].m.type = type;
+    b.job[0].m.cols = cols;
+    b.job[0].x = x;
+    b.job[0].tokens = tokens;
+    b.job[0].tok_off = 0;
+    for (uint32_t j = 1; j < MM_MAX_JOBS; j++) b.job[j] = b.job[0];
+    b.n_jobs = 1;
+    b.xb = v.xb;
+    b.sx = v.sx;
+    b.mpad = v.mpad;
+    return mm_by_type(type, [&](auto t) {
+        constexpr uint32_t T = decltype(t)::value;
+        hipLaunchKernelGGL(mm_xsplit_kernel<T>, dim3((b.mpad + XS_TOK - 1) / XS_TOK, (v.n_groups + XS_GRP - 1) / XS_GRP), dim3(256),
+                           0, stream, b, v.n_groups);
+        return hipGetLastError();
+    });
+}
+
+// The plan of n products (one dtype, one column count) of the same split activations, `tokens` tokens each.
+// forced_shares: every job writes shares (one when its columns are not shared) into the workspace, for an
+// epilogue launch to sum; otherwise jobs without shared columns write ys directly.
+static bool act_plan(const MatView *tiled, uint32_t n, uint32_t tokens, float *const *ys, bool forced_shares, MmPlan &p) {
+    if (n == 0 || n > (uint32_t)MM_MAX_JOBS || tokens < MM_MIN_TOKENS || !mm_type(tiled[0].type)) return false;
+    for (uint32_t j = 1; j < n; j++)
+        if (tiled[j].type != tiled[0].type || tiled[j].cols != tiled[0].cols) return false;
+    uint32_t toks[MM_MAX_JOBS];
+    const float *xs[MM_MAX_JOBS];
+    static const float same_x = 0.f;  // any one address: the jobs then share their split slots
+    for (uint32_t j = 0; j < n; j++) {
+        toks[j] = tokens;
+        xs[j] = &same_x;
+    }
+    mm_plan(tiled, toks, xs, ys, n, p);
+    if (forced_shares) {
+        size_t part = 0;
+        for (uint32_t j = 0; j < n; j++) {
+            const uint32_t ks = p.b.job[j].ksplit > 1 ? p.b.job[j].ksplit : 1;
+            part += up256((size_t)ks * tokens * tiled[j].rows * sizeof(float));
+        }
+        p.part_bytes = part;
+    }
+    return true;
+}
+
+size_t gemm_act_workspace_bytes(const MatView *mats, uint32_t n, uint32_t tokens, bool with_epilogue) {
+    MmPlan p;
+    if (!act_plan(mats, n, tokens, nullptr, with_epilogue, p)) return 0;
+    return p.part_bytes;
+}
+
+hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n, uint32_t tokens, void *act, uint32_t act_max_tokens,
+                           float *const *ys, const ActEpilogue &ep, void *ws, size_t ws_bytes) {
+    if (!act || tokens > act_max_tokens) return hipErrorInvalidValue;
+    const bool fused = ep.kind != ACT_EPILOGUE_NONE;
+    if (fused && (ep.kind == ACT_EPILOGUE_ADD_RMSNORM ? n != 1 : n != 2)) return hipErrorInvalidValue;
+    if (!fused && !ys) return hipErrorInvalidValue;
+    MmPlan p;
+    if (!act_plan(tiled, n, tokens, fused ? nullptr : ys, fused, p)) return hipErrorInvalidValue;
+    if (p.part_bytes > ws_bytes) return hipErrorInvalidValue;
+    MmBatch &b = p.b;
+    const ActView in = act_view(act, tiled[0].type, tiled[0].cols, act_max_tokens, tokens);
+    if (in.mpad != b.mpad) return hipErrorInvalidValue;  // the plan's slots and the buffer's must be the same thing
+    b.xb = in.xb;
+    b.sx = in.sx;
+    uint8_t *part = static_cast<uint8_t *>(ws);
+    for (uint32_t j = 0; j < b.n_jobs; j++) {
+        MmJob &job = b.job[j];
+        if (job.ksplit > 1 || fused) {
+            job.part = reinterpret_cast<float *>(part);
+            if (job.ksplit < 2) job.y = job.part;  // its one share
+            part += up256((size_t)(job.ksplit > 1 ? job.ksplit : 1) * tokens * job.m.rows * sizeof(float));
+        }
+    }
+    hipError_t e = mm_by_type(tiled[0].type, [&](auto t) {
+        constexpr uint32_t T = decltype(t)::value;
+        if constexpr (T != T_Q6_K) {
+            if (p.tile16) return launch_mm16_main<T>(stream, b);
+        }
+        if (p.tt == 2) return launch_mm_main<T, 2, 4>(stream, b);
+        if (p.max_tok <= 8) return launch_mm_main<T, 1, 1>(stream, b);
+        if (p.max_tok <= 16) return launch_mm_main<T, 1, 2>(stream, b);
+        if (p.max_tok <= 24) return launch_mm_main<T, 1, 3>(stream, b);
+        return launch_mm_main<T, 1, 4>(stream, b);
+    });
+    if (e != hipSuccess) return e;
+    if (!fused) {
+        if (b.any_split) hipLaunchKernelGGL(mm_reduce_kernel, dim3(mm_reduce_blocks(b), b.n_jobs), dim3(256), 0, stream, b);
+        return hipGetLastError();
+    }
+    ActView next{};
+    if (ep.next_act) {
+        if (act_bytes(ep.next_type, ep.next_cols, ep.next_max_tokens) == 0 || tokens > ep.next_max_tokens) return hipErrorInvalidValue;
+        next = act_view(ep.next_act, ep.next_type, ep.next_cols, ep.next_max_tokens, tokens);
+    }
+    const size_t total = (size_t)tokens * b.job[0].m.rows;
+    const uint32_t rows = b.job[0].m.rows;
+    auto shares = [&](uint32_t j) { return b.job[j].ksplit > 1 ? b.job[j].part : b.job[j].y; };
+    auto count = [&](uint32_t j) { return b.job[j].ksplit > 1 ? b.job[j].ksplit : 1u; };
+    if (ep.kind == ACT_EPILOGUE_ADD_RMSNORM) {
+        if (!ep.residual || !ep.norm_w || (ep.next_act && ep.next_cols != rows)) return hipErrorInvalidValue;
+        if ((size_t)rows * sizeof(float) > g_lds_limit) return hipErrorInvalidValue;
+        const uint32_t nt = ep.next_act ? ep.next_type : (uint32_t)T_Q8_0;
+        return mm_by_type(nt, [&](auto t) {
+            constexpr uint32_t TN = decltype(t)::value;
+            auto kern = mm_epi_add_norm_kernel<TN>;
+            const size_t lds = (size_t)rows * sizeof(float);
+            if (lds > 48 * 1024) {
+                const hipError_t a = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+                if (a != hipSuccess) return a;
+            }
+            hipLaunchKernelGGL(kern, dim3(tokens), dim3(1024), lds, stream, shares(0), count(0), total, rows, ep.residual, ep.norm_w,
+                               ep.eps, ep.xn_out, next);
+            return hipGetLastError();
+        });
+    }
+    // SiLU(gate) * up
+    if (!ep.next_act || b.job[1].m.rows != rows || ep.next_cols != rows) return hipErrorInvalidValue;
+    return mm_by_type(ep.next_type, [&](auto t) {
+        constexpr uint32_t TN = decltype(t)::value;
+        hipLaunchKernelGGL(mm_epi_swiglu_kernel<TN>, dim3((next.mpad + XS_TOK - 1) / XS_TOK, (next.n_groups + XS_GRP - 1) / XS_GRP),
+                           dim3(256), 0, stream, shares(0), count(0), shares(1), count(1), total, rows, tokens, next);
+        return hipGetLastError();
+    });
+}
+
 // Plain 16-byte-per-lane copy, used only to calibrate HBM traffic counters.
 __global__ __launch_bounds__(256) void copy_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n16) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];

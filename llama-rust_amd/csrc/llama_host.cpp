@@ -24,6 +24,7 @@
 #include <memory>
 #include <string>
 #include <thread>
+#include <map>
 #include <vector>
 
 #include <hip/hip_runtime.h>

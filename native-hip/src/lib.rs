@@ -22,6 +22,10 @@ mod ffi {
     pub struct LnhMatrix {
         _private: [u8; 0],
     }
+    #[repr(C)]
+    pub struct LnhAct {
+        _private: [u8; 0],
+    }
 
     // One declaration per entry point of include/native_hip.h that a Rust caller uses, in the
     // header's order.  `usize` is `size_t`, `u32` is `uint32_t`, `c_int` is `int`.
@@ -49,6 +53,10 @@ mod ffi {
         pub fn lnh_gemv_shared_device(exec: *mut LnhExec, n_mats: usize, mats: *const *const LnhMatrix, device_x: *const f32, device_ys: *const *mut f32, accumulate: c_int, stream: *mut c_void) -> c_int;
         pub fn lnh_gemv_fused_device(exec: *mut LnhExec, n_mats: usize, mats: *const *const LnhMatrix, device_x: *const f32, device_ys: *const *mut f32, accumulate: c_int, prologue: c_int, device_x2: *const f32, eps: f32, stream: *mut c_void) -> c_int;
         pub fn lnh_gemv_swiglu_device(exec: *mut LnhExec, gate: *const LnhMatrix, up: *const LnhMatrix, device_x: *const f32, device_h: *mut f32, prologue: c_int, device_x2: *const f32, eps: f32, stream: *mut c_void) -> c_int;
+        pub fn lnh_act_create(exec: *mut LnhExec, ggml_type: u32, cols: usize, max_tokens: usize, out: *mut *mut LnhAct) -> c_int;
+        pub fn lnh_act_free(act: *mut LnhAct);
+        pub fn lnh_act_split_device(exec: *mut LnhExec, act: *mut LnhAct, tokens: usize, device_x: *const f32, stream: *mut c_void) -> c_int;
+        pub fn lnh_gemm_act_device(exec: *mut LnhExec, n_mats: usize, mats: *const *const LnhMatrix, x: *const LnhAct, tokens: usize, device_ys: *const *mut f32, epilogue: c_int, device_residual: *mut f32, device_norm_w: *const f32, eps: f32, device_xn: *mut f32, next: *mut LnhAct, stream: *mut c_void) -> c_int;
         pub fn lnh_synchronize(exec: *mut LnhExec) -> c_int;
         pub fn lnh_shape_checked(rows: usize, cols: usize, weights_len: usize, input_len: usize, rows_out: *mut u32, cols_out: *mut u32) -> c_int;
         pub fn lnh_validate(actual: *const f32, actual_len: usize, expected: *const f64, expected_len: usize) -> c_int;

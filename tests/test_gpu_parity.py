@@ -866,3 +866,80 @@ def test_batch_entry_point_fuses_products_that_share_an_input(pkg, gpu, ty):
         b.free()
     for m in mats:
         m.close()
+
+
+@pytest.mark.parametrize("ty", [K.Q4_K, K.Q4_0, K.Q6_K, K.Q5_1, K.Q8_0])
+@pytest.mark.parametrize("tokens", [3, 16, 17, 40, 130])
+def test_split_activations_chain_equals_separate_launches(pkg, gpu, ty, tokens):
+    """lnh_act_* / lnh_gemm_act_device: a chain of three products (o-like with the residual + RMSNorm epilogue, a
+    gate/up pair with the SiLU(gate) * up epilogue, a down-like product with a plain sum) whose activations stay in
+    the split form, against the same chain through lnh_gemm_device with the element-wise steps on the host: the
+    products and the residual bit for bit (same kernels, same order of additions), the steps whose host form uses
+    other roundings (sum of squares, exp) through the next product within 2e-5 of its magnitude."""
+    import importlib
+    hip = importlib.import_module("llama-rust_amd.hiprt")
+    rng = np.random.default_rng(900 + ty * 7 + tokens)
+    d, ff = 512, 768
+    w_o, w_g, w_u, w_d = (K.random_packed(ty, r, c, rng, signed=False, scale=0.05)
+                          for r, c in ((d, d), (ff, d), (ff, d), (d, ff)))
+    m_o, m_g, m_u, m_d = (gpu.upload_packed(ty, r, c, w) for (r, c), w in (((d, d), w_o), ((ff, d), w_g), ((ff, d), w_u), ((d, ff), w_d)))
+    x0 = rng.normal(0, 1, (tokens, d)).astype(np.float32)
+    res0 = rng.normal(0, 1, (tokens, d)).astype(np.float32)
+    g = (1 + rng.normal(0, 0.05, d)).astype(np.float32)
+    eps = 1e-5
+    dev = lambda a: hip.DeviceBuffer.from_numpy(np.ascontiguousarray(a).reshape(-1))
+    d_x0, d_res, d_g = dev(x0), dev(res0), dev(g)
+    d_xn, d_y = hip.DeviceBuffer(tokens * d * 4), hip.DeviceBuffer(tokens * d * 4)
+    a_o, a_gu, a_d = gpu.act_create(ty, d, tokens + 5), gpu.act_create(ty, d, tokens), gpu.act_create(ty, ff, 2 * tokens)
+    gpu.act_split_device(a_o, tokens, d_x0.ptr)
+    gpu.gemm_act_device([m_o], a_o, tokens, None, pkg.EPILOGUE_ADD_RMSNORM, d_res.ptr, d_g.ptr, eps, d_xn.ptr, a_gu)
+    gpu.gemm_act_device([m_g, m_u], a_gu, tokens, None, pkg.EPILOGUE_SWIGLU, next_act=a_d)
+    gpu.gemm_act_device([m_d], a_d, tokens, [d_y.ptr])
+    gpu.synchronize()
+    got_res = d_res.to_numpy(np.float32).reshape(tokens, d)
+    got_xn = d_xn.to_numpy(np.float32).reshape(tokens, d)
+    got_y = d_y.to_numpy(np.float32).reshape(tokens, d)
+
+    def product(m, rows, x):
+        dx, dy = dev(x), hip.DeviceBuffer(x.shape[0] * rows * 4)
+        gpu.gemm_device(m, x.shape[0], dx.ptr, dy.ptr)
+        gpu.synchronize()
+        y = dy.to_numpy(np.float32).reshape(x.shape[0], rows)
+        dx.free(); dy.free()
+        return y
+
+    # the o-like product and the residual addition: bit for bit
+    want_res = res0 + product(m_o, d, x0)
+    assert np.array_equal(got_res, want_res)
+    # RMSNorm of the new residual: against float64
+    r64 = want_res.astype(np.float64)
+    xn64 = r64 / np.sqrt(np.mean(r64 * r64, axis=1, keepdims=True) + eps) * g.astype(np.float64)
+    assert np.abs(got_xn - xn64).max() <= 4e-6 * np.abs(xn64).max()
+    # what the gate/up pair read is the split of exactly those rows: the pair's products of got_xn, SiLU * up on
+    # the host, the down-like product of that, against the chain's result
+    gate, up = product(m_g, ff, got_xn), product(m_u, ff, got_xn)
+    with np.errstate(over="ignore"):
+        h = (gate.astype(np.float64) / (1 + np.exp(-gate.astype(np.float64))) * up.astype(np.float64)).astype(np.float32)
+    want_y = product(m_d, d, h)
+    _, mag = O.gemm_f64_mag(ty, ff, tokens, w_d, h.reshape(-1), d)
+    assert np.all(np.abs(got_y - want_y) <= 2e-5 * np.asarray(mag).reshape(tokens, d) + 1e-30), \
+        float(np.max(np.abs(got_y - want_y) / (np.asarray(mag).reshape(tokens, d) + 1e-30)))
+    # a plain sum after split activations is the three-launch product itself
+    d_y2 = hip.DeviceBuffer(tokens * ff * 4)
+    gpu.act_split_device(a_gu, tokens, dev(got_xn).ptr)
+    gpu.gemm_act_device([m_g], a_gu, tokens, [d_y2.ptr])
+    gpu.synchronize()
+    assert np.array_equal(d_y2.to_numpy(np.float32).reshape(tokens, ff), gate)
+    # refusals: fewer than three tokens, another dtype's activations, capacity
+    with pytest.raises(pkg.NativeHipError, match="three or more tokens"):
+        gpu.gemm_act_device([m_d], a_d, 2, [d_y.ptr])
+    with pytest.raises(pkg.NativeHipError, match="another dtype or column count"):
+        gpu.gemm_act_device([m_d], a_o, tokens, [d_y.ptr])
+    with pytest.raises(pkg.NativeHipError, match="capacity"):
+        gpu.act_split_device(a_gu, tokens + 1, d_x0.ptr)
+    with pytest.raises(pkg.NativeHipError, match="block-quantized"):
+        gpu.act_create(K.F16, d, tokens)
+    for a in (a_o, a_gu, a_d):
+        a.close()
+    for m in (m_o, m_g, m_u, m_d):
+        m.close()

@@ -49,7 +49,7 @@ def c_kind(decl, has_name=True):
 def base_kind(name):
     name = name.strip()
     table = {"size_t": "usize", "uint32_t": "u32", "uint8_t": "u8", "int": "int", "float": "f32", "double": "f64",
-             "char": "char", "void": "void", "lnh_exec": "exec", "lnh_matrix": "matrix"}
+             "char": "char", "void": "void", "lnh_exec": "exec", "lnh_matrix": "matrix", "lnh_act": "act"}
     if name.startswith("const "):
         name = name[6:].strip()
     assert name in table, name
@@ -62,7 +62,7 @@ def rust_kind(ty):
     if m:
         return ("ptr", m.group(1) == "const", rust_kind(m.group(2)))
     table = {"usize": "usize", "u32": "u32", "u8": "u8", "c_int": "int", "f32": "f32", "f64": "f64", "c_char": "char",
-             "c_void": "void", "LnhExec": "exec", "LnhMatrix": "matrix"}
+             "c_void": "void", "LnhExec": "exec", "LnhMatrix": "matrix", "LnhAct": "act"}
     assert ty in table, ty
     return table[ty]
 
