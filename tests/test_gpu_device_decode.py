@@ -263,6 +263,30 @@ def test_batch_session_equals_independent_sessions(pkg, llama, tmp_path, n_seq, 
     assert again[::-1].tolist() == together.tolist()
 
 
+@pytest.mark.parametrize("block_type,output_type,n_seq", [(12, 1, 8), (12, 14, 20), (1, 1, 5), (2, 0, 3)])
+def test_split_activation_chain_and_separate_launches_give_the_same_session(pkg, llama, tmp_path, monkeypatch, block_type,
+                                                                            output_type, n_seq):
+    """Multi-token steps keep their activations split between products (lnh_gemm_act_device) unless
+    LLAMA_HIP_BATCH_UNFUSED is set or a layer matrix is F16 / F32: both ways the same tokens from the batch session
+    and, for a prompt that runs as chunks, the same logits bit for bit from the device session (the fused launches
+    sum and normalise in the order of the kernels they replace).  Heads that read plain rows (F16, F32) and heads
+    that read split activations (Q6_K) both occur."""
+    path = tmp_path / "small.gguf"
+    llama.write_synthetic_llama(path, n_layer=3, n_embd=512, n_head=8, n_head_kv=2, n_ff=1536, n_vocab=2048,
+                                block_type=block_type, embd_type=block_type, output_type=output_type, seed=47)
+    m = llama.Llama(path=path)
+    rng = np.random.default_rng(7 + n_seq)
+    prompts = [rng.integers(0, 2048, int(n)).tolist() for n in rng.integers(1, 90, n_seq)]
+    long_prompt = rng.integers(0, 2048, 141).tolist()
+    chained = m.batch_session(n_seq, 128).generate_greedy(prompts, 12)[0]
+    logits_chained = m.session(device_positions=160).forward(long_prompt)
+    monkeypatch.setenv("LLAMA_HIP_BATCH_UNFUSED", "1")
+    separate = m.batch_session(n_seq, 128).generate_greedy(prompts, 12)[0]
+    logits_separate = m.session(device_positions=160).forward(long_prompt)
+    assert chained.tolist() == separate.tolist()
+    assert logits_chained.view(np.uint32).tolist() == logits_separate.view(np.uint32).tolist()
+
+
 def test_batch_session_refuses_what_it_cannot_do(pkg, llama, tmp_path):
     path = tmp_path / "small.gguf"
     llama.write_synthetic_llama(path, n_layer=2, n_embd=256, n_head=4, n_head_kv=2, n_ff=512, n_vocab=512, seed=43)
