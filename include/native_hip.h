@@ -210,7 +210,8 @@ int lnh_gemv_swiglu_device(lnh_exec *exec, const lnh_matrix *gate, const lnh_mat
  *     LNH_EPILOGUE_NONE         device_ys[i] = mats[i] x                        (any number of matrices)
  *     LNH_EPILOGUE_ADD_RMSNORM  device_residual += mats[0] x, then RMSNorm of the new residual times device_norm_w
  *                               (langtax/src/decode.rs:2957 / 3043 and 11498-11513) into device_xn (plain rows, may
- *                               be NULL) and into `next` (may be NULL), whose columns are the matrix's rows
+ *                               be NULL) and into `next` (may be NULL), whose columns are the matrix's rows;
+ *                               LNH_ERR_UNSUPPORTED for matrices of more than 12288 rows
  *     LNH_EPILOGUE_SWIGLU       SiLU(mats[0] x) * (mats[1] x) (decode.rs:11826-11830, 2981-2984) into `next`
  *   Sums run in share order and the row operations in the order of a one-workgroup-per-row kernel, so results
  *   equal those of the three-launch product followed by separate element-wise kernels bit for bit.

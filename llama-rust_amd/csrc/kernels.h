@@ -50,6 +50,7 @@ hipError_t launch_gemm_groups(hipStream_t stream, const MatView *mats, const Mat
 // ws must hold gemm_act_workspace_bytes() for the same arguments.  hipErrorInvalidValue = not this path's case,
 // nothing launched.
 enum { ACT_EPILOGUE_NONE = 0, ACT_EPILOGUE_ADD_RMSNORM = 1, ACT_EPILOGUE_SWIGLU = 2 };
+constexpr size_t ACT_NORM_MAX_ROW_BYTES = 48 * 1024;  // ADD_RMSNORM: rows of at most 12288 floats
 struct ActEpilogue {
     int kind = ACT_EPILOGUE_NONE;
     float *residual = nullptr;

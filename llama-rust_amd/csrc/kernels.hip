@@ -885,6 +885,7 @@ size_t gemm_act_workspace_bytes(const MatView *mats, uint32_t n, uint32_t tokens
 
 hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n, uint32_t tokens, void *act, uint32_t act_max_tokens,
                            float *const *ys, const ActEpilogue &ep, void *ws, size_t ws_bytes) {
+    // everything is checked before the first launch: a refusal leaves the stream as it was
     if (!act || tokens > act_max_tokens) return hipErrorInvalidValue;
     const bool fused = ep.kind != ACT_EPILOGUE_NONE;
     if (fused && (ep.kind == ACT_EPILOGUE_ADD_RMSNORM ? n != 1 : n != 2)) return hipErrorInvalidValue;
@@ -895,6 +896,21 @@ hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n,
     MmBatch &b = p.b;
     const ActView in = act_view(act, tiled[0].type, tiled[0].cols, act_max_tokens, tokens);
     if (in.mpad != b.mpad) return hipErrorInvalidValue;  // the plan's slots and the buffer's must be the same thing
+    const uint32_t rows = tiled[0].rows;
+    ActView next{};
+    if (ep.next_act) {
+        if (!fused || act_bytes(ep.next_type, ep.next_cols, ep.next_max_tokens) == 0 || tokens > ep.next_max_tokens ||
+            ep.next_cols != rows)
+            return hipErrorInvalidValue;
+        next = act_view(ep.next_act, ep.next_type, ep.next_cols, ep.next_max_tokens, tokens);
+    }
+    if (ep.kind == ACT_EPILOGUE_ADD_RMSNORM) {
+        if (!ep.residual || !ep.norm_w) return hipErrorInvalidValue;
+        // the row passes through LDS; rows beyond the default dynamic limit would need an attribute set outside captures
+        if ((size_t)rows * sizeof(float) > ACT_NORM_MAX_ROW_BYTES) return hipErrorInvalidValue;
+    }
+    if (ep.kind == ACT_EPILOGUE_SWIGLU && (!ep.next_act || tiled[1].rows != rows)) return hipErrorInvalidValue;
+
     b.xb = in.xb;
     b.sx = in.sx;
     uint8_t *part = static_cast<uint8_t *>(ws);
@@ -922,36 +938,18 @@ hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n,
         if (b.any_split) hipLaunchKernelGGL(mm_reduce_kernel, dim3(mm_reduce_blocks(b), b.n_jobs), dim3(256), 0, stream, b);
         return hipGetLastError();
     }
-    ActView next{};
-    if (ep.next_act) {
-        if (act_bytes(ep.next_type, ep.next_cols, ep.next_max_tokens) == 0 || tokens > ep.next_max_tokens) return hipErrorInvalidValue;
-        next = act_view(ep.next_act, ep.next_type, ep.next_cols, ep.next_max_tokens, tokens);
-    }
-    const size_t total = (size_t)tokens * b.job[0].m.rows;
-    const uint32_t rows = b.job[0].m.rows;
+    const size_t total = (size_t)tokens * rows;
     auto shares = [&](uint32_t j) { return b.job[j].ksplit > 1 ? b.job[j].part : b.job[j].y; };
     auto count = [&](uint32_t j) { return b.job[j].ksplit > 1 ? b.job[j].ksplit : 1u; };
-    if (ep.kind == ACT_EPILOGUE_ADD_RMSNORM) {
-        if (!ep.residual || !ep.norm_w || (ep.next_act && ep.next_cols != rows)) return hipErrorInvalidValue;
-        if ((size_t)rows * sizeof(float) > g_lds_limit) return hipErrorInvalidValue;
-        const uint32_t nt = ep.next_act ? ep.next_type : (uint32_t)T_Q8_0;
+    const uint32_t nt = ep.next_act ? ep.next_type : (uint32_t)T_Q8_0;  // without next activations the column order is never used
+    if (ep.kind == ACT_EPILOGUE_ADD_RMSNORM)
         return mm_by_type(nt, [&](auto t) {
             constexpr uint32_t TN = decltype(t)::value;
-            auto kern = mm_epi_add_norm_kernel<TN>;
-            const size_t lds = (size_t)rows * sizeof(float);
-            if (lds > 48 * 1024) {
-                const hipError_t a = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-                if (a != hipSuccess) return a;
-            }
-            hipLaunchKernelGGL(kern, dim3(tokens), dim3(1024), lds, stream, shares(0), count(0), total, rows, ep.residual, ep.norm_w,
-                               ep.eps, ep.xn_out, next);
+            hipLaunchKernelGGL(mm_epi_add_norm_kernel<TN>, dim3(tokens), dim3(1024), (size_t)rows * sizeof(float), stream, shares(0),
+                               count(0), total, rows, ep.residual, ep.norm_w, ep.eps, ep.xn_out, next);
             return hipGetLastError();
         });
-    }
-    // SiLU(gate) * up
-    if (!ep.next_act || b.job[1].m.rows != rows || ep.next_cols != rows) return hipErrorInvalidValue;
-    return mm_by_type(ep.next_type, [&](auto t) {
+    return mm_by_type(nt, [&](auto t) {  // SiLU(gate) * up
         constexpr uint32_t TN = decltype(t)::value;
         hipLaunchKernelGGL(mm_epi_swiglu_kernel<TN>, dim3((next.mpad + XS_TOK - 1) / XS_TOK, (next.n_groups + XS_GRP - 1) / XS_GRP),
                            dim3(256), 0, stream, shares(0), count(0), shares(1), count(1), total, rows, tokens, next);
