@@ -868,7 +868,7 @@ def test_batch_entry_point_fuses_products_that_share_an_input(pkg, gpu, ty):
         m.close()
 
 
-@pytest.mark.parametrize("ty", [K.Q4_K, K.Q4_0, K.Q6_K, K.Q5_1, K.Q8_0])
+@pytest.mark.parametrize("ty", [K.Q4_K, K.Q4_0, K.Q6_K, K.Q5_0, K.Q5_1, K.Q8_0])
 @pytest.mark.parametrize("tokens", [3, 16, 17, 40, 130])
 def test_split_activations_chain_equals_separate_launches(pkg, gpu, ty, tokens):
     """lnh_act_* / lnh_gemm_act_device: a chain of three products (o-like with the residual + RMSNorm epilogue, a
