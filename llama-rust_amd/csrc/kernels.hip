@@ -557,7 +557,7 @@ static hipError_t launch_mm16_main(hipStream_t stream, const MmBatch &b) {
     if constexpr (T == T_Q4_0 && !FB) {
         if (g_nibble_i4) return launch_mm16_main<T, true>(stream, b);
     }
-    constexpr size_t lds = 2 * Mm16Traits<T>::BYTES;  // two pipeline stages
+    constexpr size_t lds = Mm16Traits<T>::LDS_BYTES;  // two pipeline stages, the scale exchange
     hipLaunchKernelGGL((gemm_mfma16_kernel<T, FB>), dim3(b.total_wgs), dim3(256), lds, stream, b);
     return hipGetLastError();
 }
