@@ -478,17 +478,40 @@ static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *co
     uint32_t wgs = 0;
     bool any_split = false;
     const uint32_t n_steps = mats[0].cols / 32;
-    // Columns are shared between workgroups only as far as the row and token tiles of the whole
-    // launch leave CUs idle: every share costs a partial result written and read back.
+    // Columns are shared between workgroups as far as that shortens the launch: every share costs a partial
+    // result written and read back.  A CU holds two workgroups of these kernels, and one alone already gets 0.63-0.7
+    // of what the two get together (measured on the 16-token kernel: a step of 0.48 us alone, 0.76 us each
+    // together), so what counts is how evenly the steps fall on the CUs.  The launch is priced in steps of a
+    // workgroup that shares its CU: whole rounds of 2 x CUs workgroups, then the rest (alone on their CUs if they
+    // are at most one per CU), two more steps per workgroup for its start and end; the shares at what the launch
+    // that sums them costs (their bytes at 3 TB/s + 3.5 us).  The constants are fitted to 4096x14336 / 14336x4096
+    // products of 8 to 512 tokens and to the grouped products of a routed layer (8 experts, 9 to 21 tokens each).
     uint32_t launch_tiles = 0;
-    for (uint32_t j = 0; j < n; j++)
+    size_t share_bytes = 0;  // one share of every job
+    for (uint32_t j = 0; j < n; j++) {
         launch_tiles += ((tokens[j] + tile_tok - 1) / tile_tok) * ((mats[j].rows + MM_ROWS - 1) / MM_ROWS);
-    uint32_t ks_launch = (uint32_t)(2 * g_cu_count) / (launch_tiles ? launch_tiles : 1);  // two workgroups per CU (measured best of 1..4, both tile sizes)
-    // A share is at least 256 columns: the kernels could cut finer, but 32 shares of a 4096-column matrix cost the
-    // launch that sums them more than the 16 leave idle (8 sequences decoded together: 2110 -> 2055 tok/s).
-    if (ks_launch > n_steps / 8) ks_launch = n_steps / 8;
-    if (ks_launch > 32) ks_launch = 32;
-    if (ks_launch < 1) ks_launch = 1;
+        share_bytes += (size_t)tokens[j] * mats[j].rows * sizeof(float);
+    }
+    // a share is at least 256 columns: finer ones (32 shares of a 4096-column matrix) cost the launch that sums them
+    // more than they gain (8 sequences decoded together: 2110 -> 2055 tok/s)
+    uint32_t ks_max = n_steps / 8;
+    if (ks_max > 32) ks_max = 32;
+    if (ks_max < 1) ks_max = 1;
+    const uint32_t slots = (uint32_t)(2 * g_cu_count), alone = (uint32_t)g_cu_count;
+    const double step_us = p.tt == 2 ? 1.5 : 0.7;
+    uint32_t ks_launch = 1;
+    double best = 0.0;
+    for (uint32_t ks = 1; ks <= ks_max; ks++) {
+        const uint64_t wg = (uint64_t)(launch_tiles ? launch_tiles : 1) * ks;
+        const double len = (double)((n_steps + ks - 1) / ks) + 2.0;
+        const uint64_t rounds = wg / slots, rest = wg % slots;
+        double cost = (double)rounds * len + (rest == 0 ? 0.0 : rest <= alone ? 0.7 * len : len);
+        if (ks > 1) cost += ((double)ks * (double)share_bytes / 3.0e6 + 3.5) / step_us;
+        if (ks == 1 || cost < best) {
+            best = cost;
+            ks_launch = ks;
+        }
+    }
     for (uint32_t j = 0; j < n; j++) {
         MmJob &job = b.job[j];
         job.m = mats[j];
