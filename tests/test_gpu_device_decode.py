@@ -263,6 +263,22 @@ def test_batch_session_equals_independent_sessions(pkg, llama, tmp_path, n_seq, 
     assert again[::-1].tolist() == together.tolist()
 
 
+def test_batch_step_with_more_heads_times_rows_than_large_workgroups_fit(pkg, llama, tmp_path):
+    """A step whose heads x sequences exceed two 1024-thread workgroups per CU (32 heads x 20 sequences = 640 > 512
+    on a 256-CU part) takes the attention kernel with 256-thread workgroups, the prompt chunks' instantiation with
+    RoPE and the K/V store inside: the same tokens as every sequence decoded on its own (1024-thread kernel)."""
+    path = tmp_path / "heads.gguf"
+    llama.write_synthetic_llama(path, n_layer=2, n_embd=1024, n_head=32, n_head_kv=8, n_ff=1536, n_vocab=2048, seed=43)
+    m = llama.Llama(path=path)
+    rng = np.random.default_rng(77)
+    n_seq, n_new, cap = 20, 10, 96
+    prompts = [rng.integers(0, 2048, int(n)).tolist() for n in rng.integers(1, 70, n_seq)]
+    together, _, _ = m.batch_session(n_seq, cap).generate_greedy(prompts, n_new)
+    for b in range(n_seq):
+        alone, _, _ = m.session(device_positions=cap).generate_greedy(prompts[b], n_new)
+        assert together[b].tolist() == alone.tolist(), f"sequence {b}"
+
+
 @pytest.mark.parametrize("block_type,output_type,n_seq", [(12, 1, 8), (12, 14, 20), (1, 1, 5), (2, 0, 3)])
 def test_split_activation_chain_and_separate_launches_give_the_same_session(pkg, llama, tmp_path, monkeypatch, block_type,
                                                                             output_type, n_seq):
