@@ -572,16 +572,17 @@ static hipError_t launch_mm_main(hipStream_t stream, const MmBatch &b) {
     return hipGetLastError();
 }
 
-template <uint32_t T, bool FB = false>
+// INLINE: the jobs' x are plain f32 rows and the kernel cuts them itself (no mm_xsplit launch before it).
+template <uint32_t T, bool INLINE = false, bool FB = false>
 static hipError_t launch_mm16_main(hipStream_t stream, const MmBatch &b) {
     if constexpr (T == T_Q4_K && !FB) {
-        if (b.nibble_bf16) return launch_mm16_main<T, true>(stream, b);
+        if (b.nibble_bf16) return launch_mm16_main<T, INLINE, true>(stream, b);
     }
     if constexpr (T == T_Q4_0 && !FB) {
-        if (g_nibble_i4) return launch_mm16_main<T, true>(stream, b);
+        if (g_nibble_i4) return launch_mm16_main<T, INLINE, true>(stream, b);
     }
     constexpr size_t lds = Mm16Traits<T>::LDS_BYTES;  // two pipeline stages, the scale exchange
-    hipLaunchKernelGGL((gemm_mfma16_kernel<T, FB>), dim3(b.total_wgs), dim3(256), lds, stream, b);
+    hipLaunchKernelGGL((gemm_mfma16_kernel<T, FB, INLINE>), dim3(b.total_wgs), dim3(256), lds, stream, b);
     return hipGetLastError();
 }
 
@@ -608,17 +609,17 @@ static hipError_t launch_mm_t(hipStream_t stream, MmPlan &p, void *ws, size_t ws
             b.job[j].part = reinterpret_cast<float *>(part);
             part += up256((size_t)b.job[j].ksplit * b.job[j].tokens * b.job[j].m.rows * sizeof(float));
         }
-    hipLaunchKernelGGL(mm_xsplit_kernel<T>, dim3((b.mpad + XS_TOK - 1) / XS_TOK, (p.n_groups + XS_GRP - 1) / XS_GRP),
-                       dim3(256), 0, stream, b, p.n_groups);
     hipError_t e;
     if constexpr (T != T_Q6_K) {
-        if (p.tile16) {
-            e = launch_mm16_main<T>(stream, b);
+        if (p.tile16) {  // the 16-token kernel cuts the activations itself
+            e = launch_mm16_main<T, true>(stream, b);
             if (e != hipSuccess) return e;
             if (b.any_split) hipLaunchKernelGGL(mm_reduce_kernel, dim3(mm_reduce_blocks(b), b.n_jobs), dim3(256), 0, stream, b);
             return hipGetLastError();
         }
     }
+    hipLaunchKernelGGL(mm_xsplit_kernel<T>, dim3((b.mpad + XS_TOK - 1) / XS_TOK, (p.n_groups + XS_GRP - 1) / XS_GRP),
+                       dim3(256), 0, stream, b, p.n_groups);
     if (p.tt == 2) e = launch_mm_main<T, 2, 4>(stream, b);
     else if (p.max_tok <= 8) e = launch_mm_main<T, 1, 1>(stream, b);
     else if (p.max_tok <= 16) e = launch_mm_main<T, 1, 2>(stream, b);
