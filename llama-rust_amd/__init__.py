@@ -142,6 +142,7 @@ def load_library():
         "lnh_act_free": (None, [vp]),
         "lnh_act_split_device": (C.c_int, [vp, vp, sz, vp, vp]),
         "lnh_gemm_act_device": (C.c_int, [vp, sz, vp, vp, sz, vp, C.c_int, vp, vp, C.c_float, vp, vp, vp]),
+        "lnh_gemm_plain_act_device": (C.c_int, [vp, sz, vp, vp, sz, vp, C.c_int, vp, vp, C.c_float, vp, vp, vp]),
         "lnm_forward": (C.c_int, [vp, vp, sz, vp]),
         "lnm_prompt": (C.c_int, [vp, vp, sz, vp, vp]),
         "lnm_generate_greedy": (C.c_int, [vp, vp, sz, sz, vp, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
@@ -373,6 +374,16 @@ class HipGemv:
         self._check(self._lib.lnh_gemm_act_device(self._h, n, mats, act._h, tokens, ys, epilogue, C.c_void_p(residual_ptr),
                                                   C.c_void_p(norm_w_ptr), eps, C.c_void_p(xn_ptr),
                                                   next_act._h if next_act is not None else None, C.c_void_p(stream)))
+
+    def gemm_plain_act_device(self, matrices, x_ptr, tokens, y_ptrs=None, epilogue=EPILOGUE_NONE, residual_ptr=0, norm_w_ptr=0,
+                              eps=0.0, xn_ptr=0, next_act=None, stream=0):
+        """gemm_act_device with the product's own activations as plain f32 rows on the device."""
+        n = len(matrices)
+        mats = (C.c_void_p * n)(*[m._h for m in matrices])
+        ys = (C.c_void_p * n)(*y_ptrs) if y_ptrs is not None else None
+        self._check(self._lib.lnh_gemm_plain_act_device(self._h, n, mats, C.c_void_p(x_ptr), tokens, ys, epilogue,
+                                                        C.c_void_p(residual_ptr), C.c_void_p(norm_w_ptr), eps, C.c_void_p(xn_ptr),
+                                                        next_act._h if next_act is not None else None, C.c_void_p(stream)))
 
     def gemm_grouped_device(self, matrices, tokens, x_ptr, y_ptr, stream=0):
         n = len(matrices)

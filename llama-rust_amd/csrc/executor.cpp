@@ -691,15 +691,19 @@ int lnh_act_split_device(lnh_exec *e, lnh_act *a, size_t tokens, const float *dx
     return LNH_OK;
 }
 
-int lnh_gemm_act_device(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, const lnh_act *x, size_t tokens,
-                        float *const *dys, int epilogue, float *d_residual, const float *d_norm_w, float eps, float *d_xn,
-                        lnh_act *next, void *stream) {
+}  // extern "C"
+
+namespace {
+// lnh_gemm_act_device (x) and lnh_gemm_plain_act_device (dx): the product's activations split or plain.
+int gemm_act(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, const lnh_act *x, const float *dx, size_t tokens,
+             float *const *dys, int epilogue, float *d_residual, const float *d_norm_w, float eps, float *d_xn, lnh_act *next,
+             void *stream) {
     if (!e) return LNH_ERR_INVALID;
-    if (!mats || !x || n_mats == 0) return fail(e, LNH_ERR_INVALID, "matrix list or activations are null");
+    if (!mats || (!x && !dx) || n_mats == 0) return fail(e, LNH_ERR_INVALID, "matrix list or activations are null");
     if (n_mats > 8) return fail(e, LNH_ERR_INVALID, "at most 8 matrices per call");
-    if (x->ctx.get() != e->ctx.get() || (next && next->ctx.get() != e->ctx.get()))
+    if ((x && x->ctx.get() != e->ctx.get()) || (next && next->ctx.get() != e->ctx.get()))
         return fail(e, LNH_ERR_FOREIGN, "activations belong to a different executor");
-    if (tokens == 0 || tokens > x->max_tokens || (next && tokens > next->max_tokens))
+    if (tokens == 0 || tokens > UINT32_MAX || (x && tokens > x->max_tokens) || (next && tokens > next->max_tokens))
         return fail(e, LNH_ERR_INVALID, "token count outside the activations' capacity");
     if (tokens < nh::MM_MIN_TOKENS)
         return fail(e, LNH_ERR_UNSUPPORTED, "split activations serve products of three or more tokens");
@@ -708,8 +712,10 @@ int lnh_gemm_act_device(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mat
         const lnh_matrix *m = mats[i];
         if (!m) return fail(e, LNH_ERR_INVALID, "HIP matrix is null");
         if (m->ctx.get() != e->ctx.get()) return fail(e, LNH_ERR_FOREIGN, "HIP matrix belongs to a different executor");
-        if (m->view.type != x->type || m->view.cols != x->cols)
-            return fail(e, LNH_ERR_INVALID, "the activations were split for another dtype or column count than the matrix has");
+        if (x ? (m->view.type != x->type || m->view.cols != x->cols)
+              : (m->view.type != mats[0]->view.type || m->view.cols != mats[0]->view.cols))
+            return fail(e, LNH_ERR_INVALID, x ? "the activations were split for another dtype or column count than the matrix has"
+                                              : "matrices that share an input must have one dtype and column count");
         if (m->view.rows == 0) return fail(e, LNH_ERR_INVALID, "HIP matrix has no rows");
         views[i] = m->view;
     }
@@ -749,15 +755,34 @@ int lnh_gemm_act_device(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mat
         const int rt = ensure_tiled(e, s, mats[i], &tiled[i]);
         if (rt != LNH_OK) return rt;
     }
-    int rc = ensure_workspace(e, s, nh::gemm_act_workspace_bytes(tiled, (uint32_t)n_mats, (uint32_t)tokens, ep.kind != nh::ACT_EPILOGUE_NONE));
+    int rc = ensure_workspace(e, s, nh::gemm_act_workspace_bytes(tiled, (uint32_t)n_mats, (uint32_t)tokens,
+                                                                 ep.kind != nh::ACT_EPILOGUE_NONE, x == nullptr));
     if (rc != LNH_OK) return rc;
-    const hipError_t h = nh::launch_gemm_act(s, tiled, (uint32_t)n_mats, (uint32_t)tokens, x->dev, x->max_tokens, dys, ep, e->d_ws, e->ws_cap);
+    const hipError_t h = nh::launch_gemm_act(s, tiled, (uint32_t)n_mats, (uint32_t)tokens, x ? x->dev : nullptr,
+                                             x ? x->max_tokens : 0, x ? nullptr : dx, dys, ep, e->d_ws, e->ws_cap);
     if (h == hipErrorInvalidValue) {
         (void)hipGetLastError();
         return fail(e, LNH_ERR_UNSUPPORTED, "this product is not one the split-activation path launches");
     }
     if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
     return LNH_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int lnh_gemm_act_device(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, const lnh_act *x, size_t tokens,
+                        float *const *dys, int epilogue, float *d_residual, const float *d_norm_w, float eps, float *d_xn,
+                        lnh_act *next, void *stream) {
+    if (e && !x) return fail(e, LNH_ERR_INVALID, "matrix list or activations are null");
+    return gemm_act(e, n_mats, mats, x, nullptr, tokens, dys, epilogue, d_residual, d_norm_w, eps, d_xn, next, stream);
+}
+
+int lnh_gemm_plain_act_device(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, const float *dx, size_t tokens,
+                              float *const *dys, int epilogue, float *d_residual, const float *d_norm_w, float eps,
+                              float *d_xn, lnh_act *next, void *stream) {
+    if (e && !dx) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    return gemm_act(e, n_mats, mats, nullptr, dx, tokens, dys, epilogue, d_residual, d_norm_w, eps, d_xn, next, stream);
 }
 
 int lnh_gemm_grouped_device(lnh_exec *e, size_t n_groups, const lnh_matrix *const *mats, const size_t *tokens,

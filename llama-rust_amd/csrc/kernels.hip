@@ -903,25 +903,38 @@ static bool act_plan(const MatView *tiled, uint32_t n, uint32_t tokens, float *c
     return true;
 }
 
-size_t gemm_act_workspace_bytes(const MatView *mats, uint32_t n, uint32_t tokens, bool with_epilogue) {
+size_t gemm_act_workspace_bytes(const MatView *mats, uint32_t n, uint32_t tokens, bool with_epilogue, bool plain_x) {
     MmPlan p;
     if (!act_plan(mats, n, tokens, nullptr, with_epilogue, p)) return 0;
-    return p.part_bytes;
+    // plain activations of more than 16 tokens are cut into the workspace first
+    return p.part_bytes + (plain_x && !p.tile16 ? p.xb_bytes + p.sx_bytes : 0);
 }
 
 hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n, uint32_t tokens, void *act, uint32_t act_max_tokens,
-                           float *const *ys, const ActEpilogue &ep, void *ws, size_t ws_bytes) {
+                           const float *x_plain, float *const *ys, const ActEpilogue &ep, void *ws, size_t ws_bytes) {
     // everything is checked before the first launch: a refusal leaves the stream as it was
-    if (!act || tokens > act_max_tokens) return hipErrorInvalidValue;
+    if (x_plain ? act != nullptr : (!act || tokens > act_max_tokens)) return hipErrorInvalidValue;
     const bool fused = ep.kind != ACT_EPILOGUE_NONE;
     if (fused && (ep.kind == ACT_EPILOGUE_ADD_RMSNORM ? n != 1 : n != 2)) return hipErrorInvalidValue;
     if (!fused && !ys) return hipErrorInvalidValue;
     MmPlan p;
     if (!act_plan(tiled, n, tokens, fused ? nullptr : ys, fused, p)) return hipErrorInvalidValue;
-    if (p.part_bytes > ws_bytes) return hipErrorInvalidValue;
+    const bool cut_first = x_plain && !p.tile16;  // plain activations of more than 16 tokens: mm_xsplit into the workspace
+    const size_t split_bytes = cut_first ? p.xb_bytes + p.sx_bytes : 0;
+    if (p.part_bytes + split_bytes > ws_bytes) return hipErrorInvalidValue;
     MmBatch &b = p.b;
-    const ActView in = act_view(act, tiled[0].type, tiled[0].cols, act_max_tokens, tokens);
-    if (in.mpad != b.mpad) return hipErrorInvalidValue;  // the plan's slots and the buffer's must be the same thing
+    ActView in{};
+    if (!x_plain) {
+        in = act_view(act, tiled[0].type, tiled[0].cols, act_max_tokens, tokens);
+        if (in.mpad != b.mpad) return hipErrorInvalidValue;  // the plan's slots and the buffer's must be the same thing
+    } else {
+        for (uint32_t j = 0; j < b.n_jobs; j++) b.job[j].x = x_plain;
+        for (uint32_t j = b.n_jobs; j < (uint32_t)MM_MAX_JOBS; j++) b.job[j].x = x_plain;
+        if (cut_first) {
+            in.xb = static_cast<uint4 *>(ws);
+            in.sx = reinterpret_cast<float *>(static_cast<uint8_t *>(ws) + p.xb_bytes);
+        }
+    }
     const uint32_t rows = tiled[0].rows;
     ActView next{};
     if (ep.next_act) {
@@ -939,7 +952,7 @@ hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n,
 
     b.xb = in.xb;
     b.sx = in.sx;
-    uint8_t *part = static_cast<uint8_t *>(ws);
+    uint8_t *part = static_cast<uint8_t *>(ws) + split_bytes;
     for (uint32_t j = 0; j < b.n_jobs; j++) {
         MmJob &job = b.job[j];
         if (job.ksplit > 1 || fused) {
@@ -951,8 +964,11 @@ hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n,
     hipError_t e = mm_by_type(tiled[0].type, [&](auto t) {
         constexpr uint32_t T = decltype(t)::value;
         if constexpr (T != T_Q6_K) {
-            if (p.tile16) return launch_mm16_main<T>(stream, b);
+            if (p.tile16) return x_plain ? launch_mm16_main<T, true>(stream, b) : launch_mm16_main<T>(stream, b);
         }
+        if (cut_first)
+            hipLaunchKernelGGL(mm_xsplit_kernel<T>, dim3((b.mpad + XS_TOK - 1) / XS_TOK, (p.n_groups + XS_GRP - 1) / XS_GRP),
+                               dim3(256), 0, stream, b, p.n_groups);
         if (p.tt == 2) return launch_mm_main<T, 2, 4>(stream, b);
         if (p.max_tok <= 8) return launch_mm_main<T, 1, 1>(stream, b);
         if (p.max_tok <= 16) return launch_mm_main<T, 1, 2>(stream, b);

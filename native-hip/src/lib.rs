@@ -57,6 +57,7 @@ mod ffi {
         pub fn lnh_act_free(act: *mut LnhAct);
         pub fn lnh_act_split_device(exec: *mut LnhExec, act: *mut LnhAct, tokens: usize, device_x: *const f32, stream: *mut c_void) -> c_int;
         pub fn lnh_gemm_act_device(exec: *mut LnhExec, n_mats: usize, mats: *const *const LnhMatrix, x: *const LnhAct, tokens: usize, device_ys: *const *mut f32, epilogue: c_int, device_residual: *mut f32, device_norm_w: *const f32, eps: f32, device_xn: *mut f32, next: *mut LnhAct, stream: *mut c_void) -> c_int;
+        pub fn lnh_gemm_plain_act_device(exec: *mut LnhExec, n_mats: usize, mats: *const *const LnhMatrix, device_x: *const f32, tokens: usize, device_ys: *const *mut f32, epilogue: c_int, device_residual: *mut f32, device_norm_w: *const f32, eps: f32, device_xn: *mut f32, next: *mut LnhAct, stream: *mut c_void) -> c_int;
         pub fn lnh_synchronize(exec: *mut LnhExec) -> c_int;
         pub fn lnh_shape_checked(rows: usize, cols: usize, weights_len: usize, input_len: usize, rows_out: *mut u32, cols_out: *mut u32) -> c_int;
         pub fn lnh_validate(actual: *const f32, actual_len: usize, expected: *const f64, expected_len: usize) -> c_int;

@@ -930,6 +930,24 @@ def test_split_activations_chain_equals_separate_launches(pkg, gpu, ty, tokens):
     gpu.gemm_act_device([m_g], a_gu, tokens, [d_y2.ptr])
     gpu.synchronize()
     assert np.array_equal(d_y2.to_numpy(np.float32).reshape(tokens, ff), gate)
+    # the same chain entered with plain rows (lnh_gemm_plain_act_device: up to 16 tokens the product's launch cuts
+    # them itself, more are cut into the workspace first): the same bits as through lnh_act_split_device
+    d_res2, d_xn2, d_y3 = dev(res0), hip.DeviceBuffer(tokens * d * 4), hip.DeviceBuffer(tokens * d * 4)
+    gpu.gemm_plain_act_device([m_o], d_x0.ptr, tokens, None, pkg.EPILOGUE_ADD_RMSNORM, d_res2.ptr, d_g.ptr, eps, d_xn2.ptr, a_gu)
+    gpu.gemm_act_device([m_g, m_u], a_gu, tokens, None, pkg.EPILOGUE_SWIGLU, next_act=a_d)
+    gpu.gemm_act_device([m_d], a_d, tokens, [d_y3.ptr])
+    gpu.synchronize()
+    assert np.array_equal(d_res2.to_numpy(np.float32).reshape(tokens, d), got_res)
+    assert np.array_equal(d_xn2.to_numpy(np.float32).reshape(tokens, d), got_xn)
+    assert np.array_equal(d_y3.to_numpy(np.float32).reshape(tokens, d), got_y)
+    d_y4, d_y5 = hip.DeviceBuffer(tokens * ff * 4), hip.DeviceBuffer(tokens * ff * 4)
+    d_gxn = dev(got_xn)
+    gpu.gemm_plain_act_device([m_g, m_u], d_gxn.ptr, tokens, [d_y4.ptr, d_y5.ptr])
+    gpu.synchronize()
+    assert np.array_equal(d_y4.to_numpy(np.float32).reshape(tokens, ff), gate)
+    assert np.array_equal(d_y5.to_numpy(np.float32).reshape(tokens, ff), up)
+    with pytest.raises(pkg.NativeHipError, match="one dtype and column count"):
+        gpu.gemm_plain_act_device([m_g, m_d], d_gxn.ptr, tokens, [d_y4.ptr, d_y5.ptr])
     # refusals: fewer than three tokens, another dtype's activations, capacity
     with pytest.raises(pkg.NativeHipError, match="three or more tokens"):
         gpu.gemm_act_device([m_d], a_d, 2, [d_y.ptr])
