@@ -549,18 +549,19 @@ static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *co
     p.part_bytes = part;
 }
 
-template <uint32_t T, int TT, int VQ, bool FB = false>
+// INLINE (TT = 1): the jobs' x are plain f32 rows and the kernel cuts them itself.
+template <uint32_t T, int TT, int VQ, bool INLINE = false, bool FB = false>
 static hipError_t launch_mm_main(hipStream_t stream, const MmBatch &b) {
     // FB: the device's shortcut from nibbles to bf16 codes is usable (probed at start-up): the packed
     // fp8 convert for Q4_K, the signed 4-bit convert for Q4_0
     if constexpr (T == T_Q4_K && !FB) {
-        if (b.nibble_bf16) return launch_mm_main<T, TT, VQ, true>(stream, b);
+        if (b.nibble_bf16) return launch_mm_main<T, TT, VQ, INLINE, true>(stream, b);
     }
     if constexpr (T == T_Q4_0 && !FB) {
-        if (g_nibble_i4) return launch_mm_main<T, TT, VQ, true>(stream, b);
+        if (g_nibble_i4) return launch_mm_main<T, TT, VQ, INLINE, true>(stream, b);
     }
     constexpr size_t lds = 2 * MmStage<T, TT>::BYTES;  // two pipeline stages
-    auto kern = gemm_mfma_kernel<T, TT, VQ, FB>;
+    auto kern = gemm_mfma_kernel<T, TT, VQ, FB, INLINE>;
     static bool configured = false;
     if (lds > 48 * 1024 && !configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -618,13 +619,14 @@ static hipError_t launch_mm_t(hipStream_t stream, MmPlan &p, void *ws, size_t ws
             return hipGetLastError();
         }
     }
-    hipLaunchKernelGGL(mm_xsplit_kernel<T>, dim3((b.mpad + XS_TOK - 1) / XS_TOK, (p.n_groups + XS_GRP - 1) / XS_GRP),
-                       dim3(256), 0, stream, b, p.n_groups);
-    if (p.tt == 2) e = launch_mm_main<T, 2, 4>(stream, b);
-    else if (p.max_tok <= 8) e = launch_mm_main<T, 1, 1>(stream, b);
-    else if (p.max_tok <= 16) e = launch_mm_main<T, 1, 2>(stream, b);
-    else if (p.max_tok <= 24) e = launch_mm_main<T, 1, 3>(stream, b);
-    else e = launch_mm_main<T, 1, 4>(stream, b);
+    if (p.tt == 2) {  // 64-token tiles: the activations are cut once, by a launch of their own
+        hipLaunchKernelGGL(mm_xsplit_kernel<T>, dim3((b.mpad + XS_TOK - 1) / XS_TOK, (p.n_groups + XS_GRP - 1) / XS_GRP),
+                           dim3(256), 0, stream, b, p.n_groups);
+        e = launch_mm_main<T, 2, 4>(stream, b);
+    } else if (p.max_tok <= 8) e = launch_mm_main<T, 1, 1, true>(stream, b);
+    else if (p.max_tok <= 16) e = launch_mm_main<T, 1, 2, true>(stream, b);
+    else if (p.max_tok <= 24) e = launch_mm_main<T, 1, 3, true>(stream, b);
+    else e = launch_mm_main<T, 1, 4, true>(stream, b);
     if (e != hipSuccess) return e;
     if (b.any_split) hipLaunchKernelGGL(mm_reduce_kernel, dim3(mm_reduce_blocks(b), b.n_jobs), dim3(256), 0, stream, b);
     return hipGetLastError();
@@ -906,8 +908,8 @@ static bool act_plan(const MatView *tiled, uint32_t n, uint32_t tokens, float *c
 size_t gemm_act_workspace_bytes(const MatView *mats, uint32_t n, uint32_t tokens, bool with_epilogue, bool plain_x) {
     MmPlan p;
     if (!act_plan(mats, n, tokens, nullptr, with_epilogue, p)) return 0;
-    // plain activations of more than 16 tokens are cut into the workspace first
-    return p.part_bytes + (plain_x && !p.tile16 ? p.xb_bytes + p.sx_bytes : 0);
+    // plain activations of more than 32 tokens are cut into the workspace first
+    return p.part_bytes + (plain_x && p.tt == 2 ? p.xb_bytes + p.sx_bytes : 0);
 }
 
 hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n, uint32_t tokens, void *act, uint32_t act_max_tokens,
@@ -919,7 +921,7 @@ hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n,
     if (!fused && !ys) return hipErrorInvalidValue;
     MmPlan p;
     if (!act_plan(tiled, n, tokens, fused ? nullptr : ys, fused, p)) return hipErrorInvalidValue;
-    const bool cut_first = x_plain && !p.tile16;  // plain activations of more than 16 tokens: mm_xsplit into the workspace
+    const bool cut_first = x_plain && p.tt == 2;  // plain activations of more than 32 tokens: mm_xsplit into the workspace
     const size_t split_bytes = cut_first ? p.xb_bytes + p.sx_bytes : 0;
     if (p.part_bytes + split_bytes > ws_bytes) return hipErrorInvalidValue;
     MmBatch &b = p.b;
@@ -970,6 +972,12 @@ hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n,
             hipLaunchKernelGGL(mm_xsplit_kernel<T>, dim3((b.mpad + XS_TOK - 1) / XS_TOK, (p.n_groups + XS_GRP - 1) / XS_GRP),
                                dim3(256), 0, stream, b, p.n_groups);
         if (p.tt == 2) return launch_mm_main<T, 2, 4>(stream, b);
+        if (x_plain) {  // 32-token tiles cut plain activations themselves
+            if (p.max_tok <= 8) return launch_mm_main<T, 1, 1, true>(stream, b);
+            if (p.max_tok <= 16) return launch_mm_main<T, 1, 2, true>(stream, b);
+            if (p.max_tok <= 24) return launch_mm_main<T, 1, 3, true>(stream, b);
+            return launch_mm_main<T, 1, 4, true>(stream, b);
+        }
         if (p.max_tok <= 8) return launch_mm_main<T, 1, 1>(stream, b);
         if (p.max_tok <= 16) return launch_mm_main<T, 1, 2>(stream, b);
         if (p.max_tok <= 24) return launch_mm_main<T, 1, 3>(stream, b);
