@@ -198,7 +198,7 @@ int lnh_gemv_swiglu_device(lnh_exec *exec, const lnh_matrix *gate, const lnh_mat
 /* Activations kept in the form the multi-token kernels read, for steps that stay on the device.  No counterpart in
  * the reference, whose every product takes and returns plain f32 rows on the host (langtax/src/native_gpu.rs:124-213).
  * A multi-token product is up to three launches: the activations are cut into three bf16 parts in the matrix's column
- * order (a launch of its own for more than 16 tokens; the matrix-core launch does it for fewer), the matrix-core launch
+ * order (a launch of its own for more than 32 tokens; the matrix-core launch does it for fewer), the matrix-core launch
  * writes one partial result per share of the columns, a last launch sums the shares.
  * Between two products of a decode step lies only element-wise work; lnh_gemm_act_device does that work in the
  * launch that sums the shares and leaves its result already cut for the next matrix, so a chain of products costs
@@ -216,7 +216,7 @@ int lnh_gemv_swiglu_device(lnh_exec *exec, const lnh_matrix *gate, const lnh_mat
  *     LNH_EPILOGUE_SWIGLU       SiLU(mats[0] x) * (mats[1] x) (decode.rs:11826-11830, 2981-2984) into `next`
  *   lnh_gemm_plain_act_device  the same product and epilogues with the product's own activations as `tokens` plain
  *                         f32 rows at device_x (the first product of a chain, or one whose input another kernel of
- *                         the caller wrote: the attention output): up to 16 tokens no launch is spent on cutting them
+ *                         the caller wrote: the attention output): up to 32 tokens no launch is spent on cutting them
  *   Sums run in share order and the row operations in the order of a one-workgroup-per-row kernel, so results
  *   equal those of the three-launch product followed by separate element-wise kernels bit for bit.
  * Like lnh_gemm_device it may grow the executor's workspace and make a matrix's multi-token layout on first use;

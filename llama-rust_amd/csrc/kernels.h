@@ -63,7 +63,7 @@ struct ActEpilogue {
 size_t act_bytes(uint32_t type, uint32_t cols, uint32_t max_tokens);
 hipError_t launch_act_split(hipStream_t stream, void *act, uint32_t type, uint32_t cols, uint32_t max_tokens, uint32_t tokens,
                             const float *x);
-// x_plain (with act == nullptr): the product's own activations are `tokens` plain f32 rows; up to 16 tokens the
+// x_plain (with act == nullptr): the product's own activations are `tokens` plain f32 rows; up to 32 tokens the
 // main launch cuts them itself, more are cut into the workspace by a launch of their own first.
 size_t gemm_act_workspace_bytes(const MatView *mats, uint32_t n, uint32_t tokens, bool with_epilogue, bool plain_x = false);
 hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n, uint32_t tokens, void *act, uint32_t act_max_tokens,
