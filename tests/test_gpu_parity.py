@@ -375,6 +375,45 @@ def test_random_gemv_and_gemm_within_bounds(pkg, gpu, ty):
 
 
 @pytest.mark.parametrize("ty", [K.Q4_0, K.Q5_0, K.Q5_1, K.Q8_0, K.Q4_K, K.Q6_K], ids=lambda t: O.TYPE_NAMES[t])
+def test_multi_token_products_of_random_shapes(pkg, gpu, ty):
+    """Seeded sweep over what decides the launch of a multi-token product: rows around the 256-row tile, column
+    counts that give odd and even step counts and from none to 32 column shares, token counts on both sides of the
+    16-, 32- and 64-token tiles (the first two cut their activations themselves), alone and as grouped calls whose
+    products share launches.  Every output against the f64 product of the dequantized weights."""
+    rng = np.random.default_rng(4200 + ty)
+    unit = K.QK[ty]
+    for case in range(14):
+        rows = int(rng.choice([1, 5, 63, 64, 65, 255, 256, 257, 300, 513]))
+        cols = unit * int(rng.choice([1, 2, 3, 5, 8, 9, 16, 17, 40]) if unit == 256 else rng.choice([1, 3, 8, 16, 17, 33, 64, 130, 257]))
+        tokens = int(rng.choice([3, 4, 7, 8, 9, 15, 16, 17, 23, 31, 32, 33, 47, 64, 65, 70]))
+        w = K.random_packed(ty, rows, cols, rng)
+        m = gpu.upload_packed(ty, rows, cols, w)
+        x = rng.normal(0, 1, tokens * cols).astype(np.float32)
+        y = np.full(tokens * rows, np.nan, np.float32)
+        gpu.gemm_resident(m, tokens, x, y)
+        check(y, ty, cols, tokens, rows, w, x)
+        m.close()
+    # grouped: four matrices of one column count, token counts that fall into different tile classes
+    for case in range(4):
+        cols = unit * int(rng.choice([2, 4, 9]) if unit == 256 else rng.choice([8, 16, 33, 72]))
+        rows = [int(r) for r in rng.choice([40, 256, 257, 520], 4)]
+        toks = [int(t) for t in rng.choice([0, 3, 9, 16, 17, 30, 33, 64], 4)]
+        ws = [K.random_packed(ty, r, cols, rng) for r in rows]
+        ms = [gpu.upload_packed(ty, r, cols, w) for r, w in zip(rows, ws)]
+        x = rng.normal(0, 1, sum(toks) * cols).astype(np.float32)
+        y = np.full(sum(t * r for t, r in zip(toks, rows)), np.nan, np.float32)
+        gpu.gemm_grouped(ms, toks, x, y)
+        xo = yo = 0
+        for r, t, w in zip(rows, toks, ws):
+            if t:
+                check(y[yo:yo + t * r], ty, cols, t, r, w, x[xo:xo + t * cols])
+            xo += t * cols
+            yo += t * r
+        for m in ms:
+            m.close()
+
+
+@pytest.mark.parametrize("ty", [K.Q4_0, K.Q5_0, K.Q5_1, K.Q8_0, K.Q4_K, K.Q6_K], ids=lambda t: O.TYPE_NAMES[t])
 def test_adversarial_activations_keep_the_reference_bound(pkg, gpu, ty):
     """The multi-token kernels hand the f32 activations to the matrix cores as three bf16 numbers
     each.  That is only a faithful f32 product (the reference never rounds activations,
