@@ -214,6 +214,12 @@ int lnh_gemv_swiglu_device(lnh_exec *exec, const lnh_matrix *gate, const lnh_mat
  *                               be NULL) and into `next` (may be NULL), whose columns are the matrix's rows;
  *                               LNH_ERR_UNSUPPORTED for matrices of more than 12288 rows
  *     LNH_EPILOGUE_SWIGLU       SiLU(mats[0] x) * (mats[1] x) (decode.rs:11826-11830, 2981-2984) into `next`
+ *     LNH_EPILOGUE_ADD_RMSNORM_DEFERRED  as ADD_RMSNORM into `next` (required; device_xn must be NULL), for at most
+ *                               32 tokens (LNH_ERR_UNSUPPORTED beyond): only the addition and the rows' sums of squares
+ *                               are formed now, by many small workgroups instead of one per token, and the product
+ *                               that reads `next` scales the rows as it loads them.  device_residual and
+ *                               device_norm_w must stay as they are until that product has run, and it must be
+ *                               called with the same token count.  Same bits as ADD_RMSNORM.
  *   lnh_gemm_plain_act_device  the same product and epilogues with the product's own activations as `tokens` plain
  *                         f32 rows at device_x (the first product of a chain, or one whose input another kernel of
  *                         the caller wrote: the attention output): up to 32 tokens no launch is spent on cutting them
@@ -222,7 +228,7 @@ int lnh_gemv_swiglu_device(lnh_exec *exec, const lnh_matrix *gate, const lnh_mat
  * Like lnh_gemm_device it may grow the executor's workspace and make a matrix's multi-token layout on first use;
  * neither is possible while the stream is being captured (run the step once before capturing it). */
 typedef struct lnh_act lnh_act;
-enum { LNH_EPILOGUE_NONE = 0, LNH_EPILOGUE_ADD_RMSNORM = 1, LNH_EPILOGUE_SWIGLU = 2 };
+enum { LNH_EPILOGUE_NONE = 0, LNH_EPILOGUE_ADD_RMSNORM = 1, LNH_EPILOGUE_SWIGLU = 2, LNH_EPILOGUE_ADD_RMSNORM_DEFERRED = 3 };
 int lnh_act_create(lnh_exec *exec, uint32_t ggml_type, size_t cols, size_t max_tokens, lnh_act **out);
 void lnh_act_free(lnh_act *act);
 int lnh_act_split_device(lnh_exec *exec, lnh_act *act, size_t tokens, const float *device_x, void *stream);

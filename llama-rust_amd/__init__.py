@@ -37,7 +37,7 @@ TYPE_NAMES = {F32: "f32", F16: "f16", Q4_0: "q4_0", Q5_0: "q5_0", Q5_1: "q5_1", 
 
 OK, ERR_INVALID, ERR_DEVICE, ERR_OOM, ERR_FOREIGN, ERR_UNSUPPORTED = range(6)
 PROLOGUE_NONE, PROLOGUE_RMSNORM, PROLOGUE_SWIGLU = 0, 1, 2
-EPILOGUE_NONE, EPILOGUE_ADD_RMSNORM, EPILOGUE_SWIGLU = 0, 1, 2
+EPILOGUE_NONE, EPILOGUE_ADD_RMSNORM, EPILOGUE_SWIGLU, EPILOGUE_ADD_RMSNORM_DEFERRED = 0, 1, 2, 3
 
 
 class NativeHipError(RuntimeError):

@@ -47,8 +47,15 @@ struct lnh_matrix {
 struct lnh_act {
     std::shared_ptr<Ctx> ctx;
     void *dev = nullptr;
-    size_t bytes = 0;
+    size_t bytes = 0;  // of the split form; the partial sums of a deferred norm follow it in the allocation
     uint32_t type = 0, cols = 0, max_tokens = 0;
+    // Set by LNH_EPILOGUE_ADD_RMSNORM_DEFERRED, cleared by everything else that fills the activations: the
+    // content is RMSNorm(deferred_x rows) * deferred_w, formed by the product that reads it.  Host state, in the
+    // order of the calls that enqueue the work, like the device content it describes.
+    const float *deferred_x = nullptr, *deferred_w = nullptr;
+    float deferred_eps = 0.f;
+    uint32_t deferred_tokens = 0;
+    float *partial() const { return reinterpret_cast<float *>(static_cast<uint8_t *>(dev) + bytes); }
 };
 
 struct lnh_exec {
@@ -650,10 +657,10 @@ int lnh_act_create(lnh_exec *e, uint32_t type, size_t cols, size_t max_tokens, l
     hipError_t h = hipSetDevice(e->ctx->device);
     if (h != hipSuccess) return hip_fail(e, h, "hipSetDevice");
     void *dev = nullptr;
-    h = hipMalloc(&dev, bytes);
+    h = hipMalloc(&dev, bytes + nh::ACT_DEFER_PARTIAL_BYTES);
     if (h != hipSuccess) return hip_fail(e, h, "HIP activation allocation");
     // slots past the tokens of a call are multiplied like any other and dropped: keep them finite from the start
-    h = hipMemsetAsync(dev, 0, bytes, e->stream);
+    h = hipMemsetAsync(dev, 0, bytes + nh::ACT_DEFER_PARTIAL_BYTES, e->stream);
     const hipError_t hs = hipStreamSynchronize(e->stream);
     if (h == hipSuccess) h = hs;
     if (h != hipSuccess) {
@@ -688,6 +695,7 @@ int lnh_act_split_device(lnh_exec *e, lnh_act *a, size_t tokens, const float *dx
     hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
     const hipError_t h = nh::launch_act_split(s, a->dev, a->type, a->cols, a->max_tokens, (uint32_t)tokens, dx);
     if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
+    a->deferred_x = nullptr;
     return LNH_OK;
 }
 
@@ -707,6 +715,16 @@ int gemm_act(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, const ln
         return fail(e, LNH_ERR_INVALID, "token count outside the activations' capacity");
     if (tokens < nh::MM_MIN_TOKENS)
         return fail(e, LNH_ERR_UNSUPPORTED, "split activations serve products of three or more tokens");
+    nh::ActNorm norm;
+    if (x && x->deferred_x) {  // the rows are a residual stream whose norm this product applies as it reads them
+        if (tokens != x->deferred_tokens)
+            return fail(e, LNH_ERR_INVALID, "the activations hold a deferred norm of another token count");
+        norm.w = x->deferred_w;
+        norm.partial = x->partial();
+        norm.eps = x->deferred_eps;
+        dx = x->deferred_x;
+    }
+    const bool plain = dx != nullptr;
     nh::MatView views[8], tiled[8];
     for (size_t i = 0; i < n_mats; i++) {
         const lnh_matrix *m = mats[i];
@@ -732,6 +750,17 @@ int gemm_act(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, const ln
         if (next && next->cols != views[0].rows) return fail(e, LNH_ERR_INVALID, "next activations do not have the product's width");
         ep.kind = nh::ACT_EPILOGUE_ADD_RMSNORM;
         break;
+    case LNH_EPILOGUE_ADD_RMSNORM_DEFERRED:
+        if (n_mats != 1) return fail(e, LNH_ERR_INVALID, "the residual epilogue takes one matrix");
+        if (!d_residual || !d_norm_w || !next) return fail(e, LNH_ERR_INVALID, "buffer pointer or next activations are null");
+        if (next->cols != views[0].rows) return fail(e, LNH_ERR_INVALID, "next activations do not have the product's width");
+        if (d_xn) return fail(e, LNH_ERR_UNSUPPORTED, "a deferred norm leaves no plain normalised rows");
+        if (tokens > nh::ACT_DEFER_MAX_TOKENS)
+            return fail(e, LNH_ERR_UNSUPPORTED, "the norm is deferred for products of at most 32 tokens");
+        if (next == x) return fail(e, LNH_ERR_INVALID, "a deferred norm cannot go into the activations the product reads");
+        ep.kind = nh::ACT_EPILOGUE_ADD_DEFER;
+        ep.partial = next->partial();
+        break;
     case LNH_EPILOGUE_SWIGLU:
         if (n_mats != 2 || views[0].rows != views[1].rows) return fail(e, LNH_ERR_INVALID, "SiLU(gate) * up takes two matrices of one shape");
         if (!next) return fail(e, LNH_ERR_INVALID, "SiLU(gate) * up needs activations to leave its result in");
@@ -744,7 +773,7 @@ int gemm_act(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, const ln
     ep.norm_w = d_norm_w;
     ep.eps = eps;
     ep.xn_out = d_xn;
-    if (next) {
+    if (next && ep.kind != nh::ACT_EPILOGUE_ADD_DEFER) {
         ep.next_act = next->dev;
         ep.next_type = next->type;
         ep.next_cols = next->cols;
@@ -756,15 +785,22 @@ int gemm_act(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, const ln
         if (rt != LNH_OK) return rt;
     }
     int rc = ensure_workspace(e, s, nh::gemm_act_workspace_bytes(tiled, (uint32_t)n_mats, (uint32_t)tokens,
-                                                                 ep.kind != nh::ACT_EPILOGUE_NONE, x == nullptr));
+                                                                 ep.kind != nh::ACT_EPILOGUE_NONE, plain));
     if (rc != LNH_OK) return rc;
-    const hipError_t h = nh::launch_gemm_act(s, tiled, (uint32_t)n_mats, (uint32_t)tokens, x ? x->dev : nullptr,
-                                             x ? x->max_tokens : 0, x ? nullptr : dx, dys, ep, e->d_ws, e->ws_cap);
+    const hipError_t h = nh::launch_gemm_act(s, tiled, (uint32_t)n_mats, (uint32_t)tokens, plain ? nullptr : x->dev,
+                                             plain ? 0 : x->max_tokens, dx, norm.w ? &norm : nullptr, dys, ep, e->d_ws, e->ws_cap);
     if (h == hipErrorInvalidValue) {
         (void)hipGetLastError();
         return fail(e, LNH_ERR_UNSUPPORTED, "this product is not one the split-activation path launches");
     }
     if (h != hipSuccess) return hip_fail(e, h, "HIP kernel launch");
+    if (next) {  // what `next` holds from here on
+        const bool deferred = ep.kind == nh::ACT_EPILOGUE_ADD_DEFER;
+        next->deferred_x = deferred ? d_residual : nullptr;
+        next->deferred_w = d_norm_w;
+        next->deferred_eps = eps;
+        next->deferred_tokens = (uint32_t)tokens;
+    }
     return LNH_OK;
 }
 }  // namespace

@@ -47,16 +47,23 @@ hipError_t launch_gemm_groups(hipStream_t stream, const MatView *mats, const Mat
 //   ADD_RMSNORM (n = 1)   residual[t] += W x[t]; xn = RMSNorm(residual[t]) * norm_w -> xn_out (may be null), next_act
 //                         (may be null; next_cols = rows of W)
 //   SWIGLU (n = 2)        SiLU(W0 x[t]) * (W1 x[t]) -> next_act (next_cols = rows of W0 = rows of W1)
+//   ADD_DEFER (n = 1)     residual[t] += W x[t], and the sixteen partial sums of squares of the new row into
+//                         `partial` (16 floats per token): the normalisation itself is left to the product that
+//                         reads the residual rows next (ActNorm below), so that many small workgroups take the place
+//                         of one per token.  tokens <= ACT_DEFER_MAX_TOKENS.
 // ws must hold gemm_act_workspace_bytes() for the same arguments.  hipErrorInvalidValue = not this path's case,
 // nothing launched.
-enum { ACT_EPILOGUE_NONE = 0, ACT_EPILOGUE_ADD_RMSNORM = 1, ACT_EPILOGUE_SWIGLU = 2 };
+enum { ACT_EPILOGUE_NONE = 0, ACT_EPILOGUE_ADD_RMSNORM = 1, ACT_EPILOGUE_SWIGLU = 2, ACT_EPILOGUE_ADD_DEFER = 3 };
 constexpr size_t ACT_NORM_MAX_ROW_BYTES = 48 * 1024;  // ADD_RMSNORM: rows of at most 12288 floats
+constexpr uint32_t ACT_DEFER_MAX_TOKENS = 32;         // the products whose main launch cuts plain rows itself
+constexpr size_t ACT_DEFER_PARTIAL_BYTES = ACT_DEFER_MAX_TOKENS * 16 * sizeof(float);
 struct ActEpilogue {
     int kind = ACT_EPILOGUE_NONE;
     float *residual = nullptr;
     const float *norm_w = nullptr;
     float eps = 0.f;
     float *xn_out = nullptr;
+    float *partial = nullptr;  // ADD_DEFER
     void *next_act = nullptr;
     uint32_t next_type = 0, next_cols = 0, next_max_tokens = 0;
 };
@@ -65,9 +72,16 @@ hipError_t launch_act_split(hipStream_t stream, void *act, uint32_t type, uint32
                             const float *x);
 // x_plain (with act == nullptr): the product's own activations are `tokens` plain f32 rows; up to 32 tokens the
 // main launch cuts them itself, more are cut into the workspace by a launch of their own first.
+// norm (with x_plain, tokens <= ACT_DEFER_MAX_TOKENS): the plain rows are a residual stream an ADD_DEFER epilogue
+// left; the product reads RMSNorm(row) * w, bit for bit what ADD_RMSNORM would have left split.
+struct ActNorm {
+    const float *w = nullptr, *partial = nullptr;
+    float eps = 0.f;
+};
 size_t gemm_act_workspace_bytes(const MatView *mats, uint32_t n, uint32_t tokens, bool with_epilogue, bool plain_x = false);
 hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n, uint32_t tokens, void *act, uint32_t act_max_tokens,
-                           const float *x_plain, float *const *ys, const ActEpilogue &ep, void *ws, size_t ws_bytes);
+                           const float *x_plain, const ActNorm *norm, float *const *ys, const ActEpilogue &ep, void *ws,
+                           size_t ws_bytes);
 
 // One launch for up to 8 single-token products that read the same x and share dtype
 // and column count (q/k/v, gate/up).  hipErrorInvalidValue = not fusable this way;

@@ -13,6 +13,7 @@
 
 #include <cmath>
 #include <cstdlib>
+#include <cstring>
 #include <type_traits>
 
 #include "kernels.h"
@@ -550,18 +551,18 @@ static void mm_plan(const MatView *mats, const uint32_t *tokens, const float *co
 }
 
 // INLINE (TT = 1): the jobs' x are plain f32 rows and the kernel cuts them itself.
-template <uint32_t T, int TT, int VQ, bool INLINE = false, bool FB = false>
+template <uint32_t T, int TT, int VQ, bool INLINE = false, bool FB = false, bool NORM = false>
 static hipError_t launch_mm_main(hipStream_t stream, const MmBatch &b) {
     // FB: the device's shortcut from nibbles to bf16 codes is usable (probed at start-up): the packed
     // fp8 convert for Q4_K, the signed 4-bit convert for Q4_0
     if constexpr (T == T_Q4_K && !FB) {
-        if (b.nibble_bf16) return launch_mm_main<T, TT, VQ, INLINE, true>(stream, b);
+        if (b.nibble_bf16) return launch_mm_main<T, TT, VQ, INLINE, true, NORM>(stream, b);
     }
     if constexpr (T == T_Q4_0 && !FB) {
-        if (g_nibble_i4) return launch_mm_main<T, TT, VQ, INLINE, true>(stream, b);
+        if (g_nibble_i4) return launch_mm_main<T, TT, VQ, INLINE, true, NORM>(stream, b);
     }
     constexpr size_t lds = 2 * MmStage<T, TT>::BYTES;  // two pipeline stages
-    auto kern = gemm_mfma_kernel<T, TT, VQ, FB, INLINE>;
+    auto kern = gemm_mfma_kernel<T, TT, VQ, FB, INLINE, NORM>;
     static bool configured = false;
     if (lds > 48 * 1024 && !configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -574,16 +575,16 @@ static hipError_t launch_mm_main(hipStream_t stream, const MmBatch &b) {
 }
 
 // INLINE: the jobs' x are plain f32 rows and the kernel cuts them itself (no mm_xsplit launch before it).
-template <uint32_t T, bool INLINE = false, bool FB = false>
+template <uint32_t T, bool INLINE = false, bool FB = false, bool NORM = false>
 static hipError_t launch_mm16_main(hipStream_t stream, const MmBatch &b) {
     if constexpr (T == T_Q4_K && !FB) {
-        if (b.nibble_bf16) return launch_mm16_main<T, INLINE, true>(stream, b);
+        if (b.nibble_bf16) return launch_mm16_main<T, INLINE, true, NORM>(stream, b);
     }
     if constexpr (T == T_Q4_0 && !FB) {
-        if (g_nibble_i4) return launch_mm16_main<T, INLINE, true>(stream, b);
+        if (g_nibble_i4) return launch_mm16_main<T, INLINE, true, NORM>(stream, b);
     }
     constexpr size_t lds = Mm16Traits<T>::LDS_BYTES;  // two pipeline stages, the scale exchange
-    hipLaunchKernelGGL((gemm_mfma16_kernel<T, FB, INLINE>), dim3(b.total_wgs), dim3(256), lds, stream, b);
+    hipLaunchKernelGGL((gemm_mfma16_kernel<T, FB, INLINE, NORM>), dim3(b.total_wgs), dim3(256), lds, stream, b);
     return hipGetLastError();
 }
 
@@ -913,11 +914,13 @@ size_t gemm_act_workspace_bytes(const MatView *mats, uint32_t n, uint32_t tokens
 }
 
 hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n, uint32_t tokens, void *act, uint32_t act_max_tokens,
-                           const float *x_plain, float *const *ys, const ActEpilogue &ep, void *ws, size_t ws_bytes) {
+                           const float *x_plain, const ActNorm *norm, float *const *ys, const ActEpilogue &ep, void *ws,
+                           size_t ws_bytes) {
     // everything is checked before the first launch: a refusal leaves the stream as it was
     if (x_plain ? act != nullptr : (!act || tokens > act_max_tokens)) return hipErrorInvalidValue;
+    if (norm && (!x_plain || tokens > ACT_DEFER_MAX_TOKENS || !norm->w || !norm->partial)) return hipErrorInvalidValue;
     const bool fused = ep.kind != ACT_EPILOGUE_NONE;
-    if (fused && (ep.kind == ACT_EPILOGUE_ADD_RMSNORM ? n != 1 : n != 2)) return hipErrorInvalidValue;
+    if (fused && (ep.kind == ACT_EPILOGUE_SWIGLU ? n != 2 : n != 1)) return hipErrorInvalidValue;
     if (!fused && !ys) return hipErrorInvalidValue;
     MmPlan p;
     if (!act_plan(tiled, n, tokens, fused ? nullptr : ys, fused, p)) return hipErrorInvalidValue;
@@ -950,10 +953,18 @@ hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n,
         // the row passes through LDS; rows beyond the default dynamic limit would need an attribute set outside captures
         if ((size_t)rows * sizeof(float) > ACT_NORM_MAX_ROW_BYTES) return hipErrorInvalidValue;
     }
+    if (ep.kind == ACT_EPILOGUE_ADD_DEFER && (!ep.residual || !ep.partial || tokens > ACT_DEFER_MAX_TOKENS || ep.next_act || ep.xn_out))
+        return hipErrorInvalidValue;
     if (ep.kind == ACT_EPILOGUE_SWIGLU && (!ep.next_act || tiled[1].rows != rows)) return hipErrorInvalidValue;
+    if (norm && p.tt == 2) return hipErrorInvalidValue;  // cannot happen up to ACT_DEFER_MAX_TOKENS tokens
 
     b.xb = in.xb;
     b.sx = in.sx;
+    if (norm) {  // what the cutting kernels read in place of split activations (gemm_mfma16_kernel's NORM)
+        b.xb = reinterpret_cast<uint4 *>(const_cast<float *>(norm->w));  // read only
+        b.sx = const_cast<float *>(norm->partial);
+        std::memcpy(&b.pad0, &norm->eps, sizeof(float));
+    }
     uint8_t *part = static_cast<uint8_t *>(ws) + split_bytes;
     for (uint32_t j = 0; j < b.n_jobs; j++) {
         MmJob &job = b.job[j];
@@ -966,7 +977,16 @@ hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n,
     hipError_t e = mm_by_type(tiled[0].type, [&](auto t) {
         constexpr uint32_t T = decltype(t)::value;
         if constexpr (T != T_Q6_K) {
+            if (p.tile16 && norm) return launch_mm16_main<T, true, false, true>(stream, b);
             if (p.tile16) return x_plain ? launch_mm16_main<T, true>(stream, b) : launch_mm16_main<T>(stream, b);
+        }
+        if (norm) {
+            if constexpr (T == T_Q6_K) {  // the other dtypes take 16-token tiles up to 16 tokens
+                if (p.max_tok <= 8) return launch_mm_main<T, 1, 1, true, false, true>(stream, b);
+                if (p.max_tok <= 16) return launch_mm_main<T, 1, 2, true, false, true>(stream, b);
+            }
+            if (p.max_tok <= 24) return launch_mm_main<T, 1, 3, true, false, true>(stream, b);
+            return launch_mm_main<T, 1, 4, true, false, true>(stream, b);
         }
         if (cut_first)
             hipLaunchKernelGGL(mm_xsplit_kernel<T>, dim3((b.mpad + XS_TOK - 1) / XS_TOK, (p.n_groups + XS_GRP - 1) / XS_GRP),
@@ -992,6 +1012,11 @@ hipError_t launch_gemm_act(hipStream_t stream, const MatView *tiled, uint32_t n,
     auto shares = [&](uint32_t j) { return b.job[j].ksplit > 1 ? b.job[j].part : b.job[j].y; };
     auto count = [&](uint32_t j) { return b.job[j].ksplit > 1 ? b.job[j].ksplit : 1u; };
     const uint32_t nt = ep.next_act ? ep.next_type : (uint32_t)T_Q8_0;  // without next activations the column order is never used
+    if (ep.kind == ACT_EPILOGUE_ADD_DEFER) {
+        hipLaunchKernelGGL(mm_epi_add_partial_kernel, dim3(tokens, 4), dim3(256), 0, stream, shares(0), count(0), total, rows,
+                           ep.residual, ep.partial);
+        return hipGetLastError();
+    }
     if (ep.kind == ACT_EPILOGUE_ADD_RMSNORM)
         return mm_by_type(nt, [&](auto t) {
             constexpr uint32_t TN = decltype(t)::value;

@@ -908,7 +908,7 @@ def test_batch_entry_point_fuses_products_that_share_an_input(pkg, gpu, ty):
 
 
 @pytest.mark.parametrize("ty", [K.Q4_K, K.Q4_0, K.Q6_K, K.Q5_0, K.Q5_1, K.Q8_0])
-@pytest.mark.parametrize("tokens", [3, 16, 17, 40, 130])
+@pytest.mark.parametrize("tokens", [3, 8, 16, 17, 24, 32, 40, 130])
 def test_split_activations_chain_equals_separate_launches(pkg, gpu, ty, tokens):
     """lnh_act_* / lnh_gemm_act_device: a chain of three products (o-like with the residual + RMSNorm epilogue, a
     gate/up pair with the SiLU(gate) * up epilogue, a down-like product with a plain sum) whose activations stay in
@@ -987,6 +987,38 @@ def test_split_activations_chain_equals_separate_launches(pkg, gpu, ty, tokens):
     assert np.array_equal(d_y5.to_numpy(np.float32).reshape(tokens, ff), up)
     with pytest.raises(pkg.NativeHipError, match="one dtype and column count"):
         gpu.gemm_plain_act_device([m_g, m_d], d_gxn.ptr, tokens, [d_y4.ptr, d_y5.ptr])
+    # the residual epilogue with its norm left to the reading product (up to 32 tokens): o-like -> gate/up -> down-like
+    # -> a gate product of the second norm, the same bits as with the norm formed in the epilogue
+    a_n = gpu.act_create(ty, d, tokens + 1)
+    d_y6, d_y7 = hip.DeviceBuffer(tokens * ff * 4), hip.DeviceBuffer(tokens * ff * 4)
+    d_res4 = dev(res0)
+    gpu.gemm_plain_act_device([m_o], d_x0.ptr, tokens, None, pkg.EPILOGUE_ADD_RMSNORM, d_res4.ptr, d_g.ptr, eps, 0, a_gu)
+    gpu.gemm_act_device([m_g, m_u], a_gu, tokens, None, pkg.EPILOGUE_SWIGLU, next_act=a_d)
+    gpu.gemm_act_device([m_d], a_d, tokens, None, pkg.EPILOGUE_ADD_RMSNORM, d_res4.ptr, d_g.ptr, eps, 0, a_n)
+    gpu.gemm_act_device([m_g], a_n, tokens, [d_y6.ptr])
+    gpu.synchronize()
+    if tokens <= 32:
+        d_res3 = dev(res0)
+        gpu.gemm_plain_act_device([m_o], d_x0.ptr, tokens, None, pkg.EPILOGUE_ADD_RMSNORM_DEFERRED, d_res3.ptr, d_g.ptr, eps, 0, a_gu)
+        gpu.gemm_act_device([m_g, m_u], a_gu, tokens, None, pkg.EPILOGUE_SWIGLU, next_act=a_d)
+        gpu.gemm_act_device([m_d], a_d, tokens, None, pkg.EPILOGUE_ADD_RMSNORM_DEFERRED, d_res3.ptr, d_g.ptr, eps, 0, a_n)
+        gpu.gemm_act_device([m_g], a_n, tokens, [d_y7.ptr])
+        gpu.synchronize()
+        assert np.array_equal(d_res3.to_numpy(np.float32), d_res4.to_numpy(np.float32))
+        assert np.array_equal(d_y7.to_numpy(np.float32), d_y6.to_numpy(np.float32))
+        with pytest.raises(pkg.NativeHipError, match="another token count"):
+            gpu.gemm_act_device([m_g], a_n, tokens + 1, [d_y7.ptr])
+        with pytest.raises(pkg.NativeHipError, match="no plain normalised rows"):
+            gpu.gemm_act_device([m_d], a_d, tokens, None, pkg.EPILOGUE_ADD_RMSNORM_DEFERRED, d_res3.ptr, d_g.ptr, eps, d_xn.ptr, a_n)
+        # filling the activations any other way ends the deferral
+        gpu.act_split_device(a_n, tokens, d_gxn.ptr)
+        gpu.gemm_act_device([m_g], a_n, tokens, [d_y7.ptr])
+        gpu.synchronize()
+        assert np.array_equal(d_y7.to_numpy(np.float32).reshape(tokens, ff), gate)
+    else:
+        with pytest.raises(pkg.NativeHipError, match="at most 32 tokens"):
+            gpu.gemm_act_device([m_d], a_d, tokens, None, pkg.EPILOGUE_ADD_RMSNORM_DEFERRED, d_res4.ptr, d_g.ptr, eps, 0, a_n)
+    a_n.close()
     # refusals: fewer than three tokens, another dtype's activations, capacity
     with pytest.raises(pkg.NativeHipError, match="three or more tokens"):
         gpu.gemm_act_device([m_d], a_d, 2, [d_y.ptr])
