@@ -907,6 +907,44 @@ def test_batch_entry_point_fuses_products_that_share_an_input(pkg, gpu, ty):
         m.close()
 
 
+@pytest.mark.parametrize("ty", [K.Q4_K, K.Q6_K, K.Q8_0])
+@pytest.mark.parametrize("tokens", [5, 20])
+def test_deferred_norm_of_zero_rows_without_eps(pkg, gpu, ty, tokens):
+    """LNH_EPILOGUE_ADD_RMSNORM_DEFERRED where the factor has its special case: a residual row that stays zero with
+    eps = 0 (rms = 0: the row is scaled by 0, decode.rs:11498-11513), next to rows of very different magnitude; the
+    reading product equals the one after LNH_EPILOGUE_ADD_RMSNORM bit for bit, and the zero row's outputs are 0."""
+    import importlib
+    hip = importlib.import_module("llama-rust_amd.hiprt")
+    rng = np.random.default_rng(1300 + ty * 5 + tokens)
+    d, ff = 1024, 256
+    w_o, w_g = K.random_packed(ty, d, d, rng, signed=True, scale=0.05), K.random_packed(ty, ff, d, rng, signed=True, scale=0.05)
+    m_o, m_g = gpu.upload_packed(ty, d, d, w_o), gpu.upload_packed(ty, ff, d, w_g)
+    x0 = rng.normal(0, 1, (tokens, d)).astype(np.float32)
+    res0 = (rng.normal(0, 1, (tokens, d)) * np.logspace(-6, 6, tokens)[:, None]).astype(np.float32)
+    x0[1] = 0
+    res0[1] = 0
+    g = (1 + rng.normal(0, 0.05, d)).astype(np.float32)
+    dev = lambda a: hip.DeviceBuffer.from_numpy(np.ascontiguousarray(a).reshape(-1))
+    d_x0, d_g = dev(x0), dev(g)
+    a_n = gpu.act_create(ty, d, tokens)
+    outs = []
+    for epilogue in (pkg.EPILOGUE_ADD_RMSNORM, pkg.EPILOGUE_ADD_RMSNORM_DEFERRED):
+        d_res, d_y = dev(res0), hip.DeviceBuffer(tokens * ff * 4)
+        gpu.gemm_plain_act_device([m_o], d_x0.ptr, tokens, None, epilogue, d_res.ptr, d_g.ptr, 0.0, 0, a_n)
+        gpu.gemm_act_device([m_g], a_n, tokens, [d_y.ptr])
+        gpu.synchronize()
+        outs.append((d_res.to_numpy(np.float32), d_y.to_numpy(np.float32).reshape(tokens, ff)))
+        d_res.free(); d_y.free()
+    assert np.array_equal(outs[0][0], outs[1][0])
+    assert np.array_equal(outs[0][1], outs[1][1])
+    assert np.all(np.isfinite(outs[1][1])) and not np.any(outs[1][1][1]) and np.any(outs[1][1][0])
+    a_n.close()
+    for m in (m_o, m_g):
+        m.close()
+    for b in (d_x0, d_g):
+        b.free()
+
+
 @pytest.mark.parametrize("ty", [K.Q4_K, K.Q4_0, K.Q6_K, K.Q5_0, K.Q5_1, K.Q8_0])
 @pytest.mark.parametrize("tokens", [3, 8, 16, 17, 24, 32, 40, 130])
 def test_split_activations_chain_equals_separate_launches(pkg, gpu, ty, tokens):
