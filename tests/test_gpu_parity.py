@@ -511,7 +511,8 @@ def test_config1_q8_0_gemv_4096(pkg, gpu):
     m.close()
 
 
-@pytest.mark.parametrize("rows,cols", [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("rows,cols", [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (4093, 14336), (13, 14336),
+                                       (8, 14336), (1, 14336), (6150, 14336)])
 def test_config2_q4_k_decode_shapes(pkg, gpu, rows, cols):
     rng = np.random.default_rng(rows + cols)
     w = _baseline_matrix(K.Q4_K, rows, cols, rng)
@@ -687,7 +688,7 @@ def test_shared_input_products_equal_separate_calls(pkg, gpu):
     """q, k, v (and gate, up) read the same activations: one call, one input copy.  The values are those
     of the separate calls bit for bit (same kernels, same order of additions within each row)."""
     rng = np.random.default_rng(21)
-    for ty, cols, rows_list in [(K.Q4_K, 4096, (4096, 1024, 1024)), (K.Q8_0, 1024, (256, 96)),
+    for ty, cols, rows_list in [(K.Q4_K, 4096, (4096, 1024, 1024)), (K.Q4_K, 14336, (100, 37, 4099)), (K.Q8_0, 1024, (256, 96)),
                                 (K.Q6_K, 512, (64, 64, 64, 64)), (K.F16, 320, (33, 7))]:
         ws = [K.random_packed(ty, r, cols, rng) for r in rows_list]
         mats = [gpu.upload_packed(ty, r, cols, w) for r, w in zip(rows_list, ws)]
