@@ -263,12 +263,15 @@ def test_batch_session_equals_independent_sessions(pkg, llama, tmp_path, n_seq, 
     assert again[::-1].tolist() == together.tolist()
 
 
-def test_batch_step_with_more_heads_times_rows_than_large_workgroups_fit(pkg, llama, tmp_path):
+@pytest.mark.parametrize("n_embd,n_head_kv", [(1024, 8), (4096, 8), (1024, 16), (1024, 32)])
+def test_batch_step_with_more_heads_times_rows_than_large_workgroups_fit(pkg, llama, tmp_path, n_embd, n_head_kv):
     """A step whose heads x sequences exceed two 1024-thread workgroups per CU (32 heads x 20 sequences = 640 > 512
-    on a 256-CU part) takes the attention kernel with 256-thread workgroups, the prompt chunks' instantiation with
-    RoPE and the K/V store inside: the same tokens as every sequence decoded on its own (1024-thread kernel)."""
+    on a 256-CU part) takes, where four query heads share a K/V head, the attention kernel with one workgroup per
+    K/V head and sequence (head sizes 32 and 128), otherwise the one with 256-thread workgroups, the prompt chunks'
+    instantiation with RoPE and the K/V store inside: the same tokens as every sequence decoded on its own
+    (1024-thread kernel)."""
     path = tmp_path / "heads.gguf"
-    llama.write_synthetic_llama(path, n_layer=2, n_embd=1024, n_head=32, n_head_kv=8, n_ff=1536, n_vocab=2048, seed=43)
+    llama.write_synthetic_llama(path, n_layer=2, n_embd=n_embd, n_head=32, n_head_kv=n_head_kv, n_ff=1536, n_vocab=2048, seed=43)
     m = llama.Llama(path=path)
     rng = np.random.default_rng(77)
     n_seq, n_new, cap = 20, 10, 96
