@@ -143,7 +143,9 @@ int lnh_gemm_shared(lnh_exec *exec, size_t n_mats, const lnh_matrix *const *mats
  * before capturing; a workspace that captured launches point at stays
  * allocated until the executor is destroyed, also after a later call has
  * made the executor move to a larger one).  Calls of one executor must therefore be enqueued on
- * one stream at a time; calls that overlap on different streams race on it. */
+ * one stream at a time; calls that overlap on different streams race on it.
+ * Every device buffer a call reads (device_x, device_x2, device_residual, device_norm_w; in this and the following
+ * sections) must be 16-byte aligned, as anything hipMalloc returns is: LNH_ERR_INVALID otherwise. */
 int lnh_gemm_device(lnh_exec *exec, const lnh_matrix *matrix, size_t tokens, const float *device_x,
                     float *device_y, void *stream);
 int lnh_gemm_grouped_device(lnh_exec *exec, size_t n_groups, const lnh_matrix *const *mats,

@@ -79,6 +79,9 @@ int fail(lnh_exec *e, int code, const std::string &msg) {
     return code;
 }
 
+// The kernels read activations, norm weights and residual rows in 16-byte pieces.
+bool misaligned(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
+
 int hip_fail(lnh_exec *e, hipError_t h, const char *what) {
     (void)hipGetLastError();  // clear the sticky error so the executor stays usable
     int code = h == hipErrorOutOfMemory ? LNH_ERR_OOM : LNH_ERR_DEVICE;
@@ -615,6 +618,7 @@ int lnh_gemm_device(lnh_exec *e, const lnh_matrix *m, size_t tokens, const float
     int rc = check_gemm(e, m, tokens, false, 0, 0, &inputs, &outputs);
     if (rc != LNH_OK) return rc;
     if (!dx || !dy) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    if (misaligned(dx)) return fail(e, LNH_ERR_INVALID, "device input buffers must be 16-byte aligned");
     hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
     return launch_products(e, s, 1, &m, &tokens, &dx, &dy);
 }
@@ -624,6 +628,7 @@ int lnh_gemm_device_noalloc(lnh_exec *e, const lnh_matrix *m, size_t tokens, con
     int rc = check_gemm(e, m, tokens, false, 0, 0, &inputs, &outputs);
     if (rc != LNH_OK) return rc;
     if (!dx || !dy) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    if (misaligned(dx)) return fail(e, LNH_ERR_INVALID, "device input buffers must be 16-byte aligned");
     void *ws = nh::static_scratch(e->ctx->device);
     if (!ws) return fail(e, LNH_ERR_DEVICE, "static workspace of this device was not initialised");
     const uint32_t tok32 = (uint32_t)tokens;
@@ -690,6 +695,7 @@ void lnh_act_free(lnh_act *a) {
 int lnh_act_split_device(lnh_exec *e, lnh_act *a, size_t tokens, const float *dx, void *stream) {
     if (!e) return LNH_ERR_INVALID;
     if (!a || !dx) return fail(e, LNH_ERR_INVALID, "activation or buffer pointer is null");
+    if (misaligned(dx)) return fail(e, LNH_ERR_INVALID, "device input buffers must be 16-byte aligned");
     if (a->ctx.get() != e->ctx.get()) return fail(e, LNH_ERR_FOREIGN, "activations belong to a different executor");
     if (tokens == 0 || tokens > a->max_tokens) return fail(e, LNH_ERR_INVALID, "token count outside the activations' capacity");
     hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
@@ -708,6 +714,7 @@ int gemm_act(lnh_exec *e, size_t n_mats, const lnh_matrix *const *mats, const ln
              void *stream) {
     if (!e) return LNH_ERR_INVALID;
     if (!mats || (!x && !dx) || n_mats == 0) return fail(e, LNH_ERR_INVALID, "matrix list or activations are null");
+    if (misaligned(dx) || misaligned(d_residual) || misaligned(d_norm_w)) return fail(e, LNH_ERR_INVALID, "device input buffers must be 16-byte aligned");
     if (n_mats > 8) return fail(e, LNH_ERR_INVALID, "at most 8 matrices per call");
     if ((x && x->ctx.get() != e->ctx.get()) || (next && next->ctx.get() != e->ctx.get()))
         return fail(e, LNH_ERR_FOREIGN, "activations belong to a different executor");
@@ -828,6 +835,7 @@ int lnh_gemm_grouped_device(lnh_exec *e, size_t n_groups, const lnh_matrix *cons
     if (rc != LNH_OK) return rc;
     if (yt == 0) return LNH_OK;
     if (!dx || !dy) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    if (misaligned(dx)) return fail(e, LNH_ERR_INVALID, "device input buffers must be 16-byte aligned");
     hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
     std::vector<const float *> xs(n_groups);
     std::vector<float *> ys(n_groups);
@@ -850,6 +858,7 @@ int lnh_gemm_batch_device(lnh_exec *e, size_t n, const lnh_matrix *const *mats, 
         int rc = check_gemm(e, mats[i], tokens[i], false, 0, 0, &inputs, &outputs);
         if (rc != LNH_OK) return rc;
         if (!dx[i] || !dy[i]) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+        if (misaligned(dx[i])) return fail(e, LNH_ERR_INVALID, "device input buffers must be 16-byte aligned");
     }
     hipStream_t s = stream ? static_cast<hipStream_t>(stream) : e->stream;
     for (size_t i = 0; i < n;) {
@@ -892,6 +901,7 @@ static int gemv_shared_device(lnh_exec *e, size_t n_mats, const lnh_matrix *cons
     if (prologue != LNH_PROLOGUE_NONE && prologue != LNH_PROLOGUE_RMSNORM && prologue != LNH_PROLOGUE_SWIGLU)
         return fail(e, LNH_ERR_INVALID, "unknown prologue");
     if (prologue != LNH_PROLOGUE_NONE && !dx2) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    if (misaligned(dx) || misaligned(dx2)) return fail(e, LNH_ERR_INVALID, "device input buffers must be 16-byte aligned");
     nh::MatView views[8];
     float *ys[8];
     for (size_t i = 0; i < n_mats; i++) {
@@ -933,6 +943,7 @@ int lnh_gemv_swiglu_device(lnh_exec *e, const lnh_matrix *gate, const lnh_matrix
     if (!dx || !dh) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
     if (prologue != LNH_PROLOGUE_NONE && prologue != LNH_PROLOGUE_RMSNORM) return fail(e, LNH_ERR_INVALID, "unknown prologue");
     if (prologue != LNH_PROLOGUE_NONE && !dx2) return fail(e, LNH_ERR_INVALID, "buffer pointer is null");
+    if (misaligned(dx) || misaligned(dx2)) return fail(e, LNH_ERR_INVALID, "device input buffers must be 16-byte aligned");
     size_t inputs, outputs;
     int rc = check_gemm(e, gate, 1, false, 0, 0, &inputs, &outputs);
     if (rc == LNH_OK) rc = check_gemm(e, up, 1, false, 0, 0, &inputs, &outputs);

@@ -149,6 +149,20 @@ def test_executor_rejects_bad_calls_and_recovers(pkg, gpu):
     free, total = gpu.memory_info()
     assert 0 < free <= total
     m.close()
+    # device buffers a call reads are taken in 16-byte pieces: an address that is not a multiple of 16 is refused
+    # before anything is launched, for one token and for several
+    import importlib
+    hip = importlib.import_module("llama-rust_amd.hiprt")
+    rng = np.random.default_rng(3)
+    mq = gpu.upload_packed(K.Q8_0, 64, 256, K.random_packed(K.Q8_0, 64, 256, rng))
+    dx, dy = hip.DeviceBuffer(8 * 256 * 4 + 16), hip.DeviceBuffer(8 * 64 * 4)
+    for tokens in (1, 8):
+        with pytest.raises(pkg.NativeHipError, match="16-byte aligned") as ei:
+            gpu.gemm_device(mq, tokens, dx.ptr + 4, dy.ptr)
+        assert ei.value.code == pkg.ERR_INVALID
+    with pytest.raises(pkg.NativeHipError, match="16-byte aligned"):
+        gpu.gemv_shared_device([mq], dx.ptr + 8, [dy.ptr])
+    mq.close(); dx.free(); dy.free()
 
 
 # ------------------------------------------------------------------ langtax/tests/native_cuda_parity.rs
