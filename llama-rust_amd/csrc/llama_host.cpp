@@ -343,6 +343,22 @@ struct MoeScratch {
     std::vector<float> logits, sel_w, pack_x, g, u, y;
     std::vector<uint32_t> sel_e, order;
     std::vector<std::vector<uint32_t>> buckets;
+    // Resident route: the packed rows go to the device once and gate, up, SiLU(gate) * up and down follow each
+    // other there (moe_ffn); grow-only buffers and a stream of the scratch's own.
+    float *d_x = nullptr, *d_g = nullptr, *d_u = nullptr, *d_y = nullptr;
+    float *h_x = nullptr, *h_y = nullptr;  // pinned: the packed rows and the down outputs on the host side of the copies
+    size_t cap_x = 0, cap_g = 0, cap_u = 0, cap_y = 0, cap_hx = 0, cap_hy = 0;  // floats
+    hipStream_t stream = nullptr;
+    MoeScratch() = default;
+    MoeScratch(const MoeScratch &) = delete;
+    MoeScratch &operator=(const MoeScratch &) = delete;
+    ~MoeScratch() {
+        for (float *p : {d_x, d_g, d_u, d_y})
+            if (p) (void)hipFree(p);
+        for (float *p : {h_x, h_y})
+            if (p) (void)hipHostFree(p);
+        if (stream) (void)hipStreamDestroy(stream);
+    }
 };
 
 }  // namespace
@@ -360,6 +376,7 @@ struct lnm_model {
     lnm_matmul_fn fn = nullptr;
     void *user = nullptr;
     lnh_exec *exec = nullptr;
+    std::unique_ptr<MoeScratch> moe_entry;  // lnm_moe_ffn's scratch
 
     ~lnm_model() {
         auto drop = [](Mat &m) {
@@ -679,6 +696,63 @@ int expert_products(lnm_model *m, std::vector<Mat> &parts, const std::vector<siz
 //   swiglu_expert_gemm 10148-10261    gate and up products, SiLU(gate) * up, down product
 //   scatter_expert_rows 10263-10292   ffn_out[t] += y[i] * w(t, e)
 // x: n x n_embd rows (already normed), ffn_out: n x n_embd, overwritten.
+__global__ void dd_swiglu_kernel(float *gate, const float *up, uint32_t n);  // with the device session's kernels below
+
+// gate, up, SiLU(gate) * up and down of every non-empty expert with the packed rows uploaded once and nothing
+// but the down outputs coming back: three grouped launches and one element-wise kernel on one stream
+// (decode.rs:10148-10261 without its host round trips between the products).
+int expert_ffn_on_device(lnm_model *m, Layer &l, const std::vector<size_t> &counts, size_t pairs, MoeScratch *ms,
+                         lnm_session *timed) {
+    const auto t0 = wall_clock::now();
+    const size_t d = m->hp.n_embd, ff = l.gate_e[0].n_rows;
+    std::vector<const lnh_matrix *> hg, hu, hd;
+    std::vector<size_t> toks;
+    for (size_t e = 0; e < counts.size(); e++) {
+        if (counts[e] == 0) continue;
+        if (ensure_resident(m, l.gate_e[e]) != 0 || ensure_resident(m, l.up_e[e]) != 0 || ensure_resident(m, l.down_e[e]) != 0)
+            return 1;
+        hg.push_back(l.gate_e[e].resident);
+        hu.push_back(l.up_e[e].resident);
+        hd.push_back(l.down_e[e].resident);
+        toks.push_back(counts[e]);
+    }
+    if (pairs * ff > UINT32_MAX) return fail("routed feed-forward: too many expert rows for one call");
+    auto grow = [&](float **p, size_t *cap, size_t want) {
+        if (*cap >= want) return hipSuccess;
+        if (*p) (void)hipFree(*p);
+        *p = nullptr;
+        *cap = 0;
+        const hipError_t e = hipMalloc(reinterpret_cast<void **>(p), want * sizeof(float));
+        if (e == hipSuccess) *cap = want;
+        return e;
+    };
+    hipError_t e = ms->stream ? hipSuccess : hipStreamCreateWithFlags(&ms->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = grow(&ms->d_x, &ms->cap_x, pairs * d);
+    if (e == hipSuccess) e = grow(&ms->d_g, &ms->cap_g, pairs * ff);
+    if (e == hipSuccess) e = grow(&ms->d_u, &ms->cap_u, pairs * ff);
+    if (e == hipSuccess) e = grow(&ms->d_y, &ms->cap_y, pairs * d);
+    if (e == hipSuccess) e = hipMemcpyAsync(ms->d_x, ms->h_x, pairs * d * sizeof(float), hipMemcpyHostToDevice, ms->stream);
+    if (e != hipSuccess) return fail(std::string("routed feed-forward: ") + hipGetErrorString(e));
+    if (lnh_gemm_grouped_device(m->exec, hg.size(), hg.data(), toks.data(), ms->d_x, ms->d_g, ms->stream) != 0 ||
+        lnh_gemm_grouped_device(m->exec, hu.size(), hu.data(), toks.data(), ms->d_x, ms->d_u, ms->stream) != 0)
+        return fail(std::string(lnh_last_error(m->exec)) + " (" + l.gate_e[0].name + ")");
+    const uint32_t n_h = (uint32_t)(pairs * ff);
+    hipLaunchKernelGGL(dd_swiglu_kernel, dim3((n_h + 1023) / 1024 < 4096 ? (n_h + 1023) / 1024 : 4096), dim3(256), 0, ms->stream,
+                       ms->d_g, ms->d_u, n_h);
+    e = hipGetLastError();
+    if (e != hipSuccess) return fail(std::string("routed feed-forward: ") + hipGetErrorString(e));
+    if (lnh_gemm_grouped_device(m->exec, hd.size(), hd.data(), toks.data(), ms->d_g, ms->d_y, ms->stream) != 0)
+        return fail(std::string(lnh_last_error(m->exec)) + " (" + l.down_e[0].name + ")");
+    e = hipMemcpyAsync(ms->h_y, ms->d_y, pairs * d * sizeof(float), hipMemcpyDeviceToHost, ms->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ms->stream);
+    if (e != hipSuccess) return fail(std::string("routed feed-forward: ") + hipGetErrorString(e));
+    if (timed) {
+        timed->products_s += since(t0);
+        timed->n_products += 3 * toks.size();
+    }
+    return 0;
+}
+
 int moe_ffn(lnm_model *m, Layer &l, size_t n, const float *x, float *ffn_out, MoeScratch *ms, lnm_session *timed) {
     const lnm_hparams &hp = m->hp;
     const size_t d = hp.n_embd, ne = hp.n_expert, k = hp.n_expert_used, ff = l.gate_e[0].n_rows;
@@ -707,22 +781,50 @@ int moe_ffn(lnm_model *m, Layer &l, size_t n, const float *x, float *ffn_out, Mo
     std::vector<size_t> counts(ne);
     size_t pairs = 0;
     for (size_t e = 0; e < ne; e++) pairs += counts[e] = ms->buckets[e].size();
+    // LLAMA_HIP_MOE_HOST_SWIGLU set: every projection a grouped call of its own through host buffers, SiLU * up on
+    // the host, as the reference's seam does it
+    const bool host_swiglu = std::getenv("LLAMA_HIP_MOE_HOST_SWIGLU") != nullptr;  // read per call: tests switch it
+    const bool on_device = m->route == LNM_PRODUCTS_RESIDENT && !host_swiglu && pairs != 0;
+    float *packed = nullptr, *expert_y = nullptr;
+    if (on_device) {
+        auto grow_pinned = [](float **p, size_t *cap, size_t want) {
+            if (*cap >= want) return hipSuccess;
+            if (*p) (void)hipHostFree(*p);
+            *p = nullptr;
+            *cap = 0;
+            const hipError_t e = hipHostMalloc(reinterpret_cast<void **>(p), want * sizeof(float), hipHostMallocDefault);
+            if (e == hipSuccess) *cap = want;
+            return e;
+        };
+        hipError_t e = grow_pinned(&ms->h_x, &ms->cap_hx, pairs * d);
+        if (e == hipSuccess) e = grow_pinned(&ms->h_y, &ms->cap_hy, pairs * d);
+        if (e != hipSuccess) return fail(std::string("routed feed-forward: ") + hipGetErrorString(e));
+        packed = ms->h_x;
+        expert_y = ms->h_y;
+    } else {
+        ms->pack_x.resize(pairs * d);
+        ms->y.resize(pairs * d);
+        packed = ms->pack_x.data();
+        expert_y = ms->y.data();
+    }
     // every expert's rows, expert after expert in ascending order
-    ms->pack_x.resize(pairs * d);
-    ms->g.resize(pairs * ff);
-    ms->u.resize(pairs * ff);
-    ms->y.resize(pairs * d);
     size_t at = 0;
     for (size_t e = 0; e < ne; e++)
-        for (uint32_t t : ms->buckets[e]) std::memcpy(&ms->pack_x[at++ * d], x + (size_t)t * d, d * sizeof(float));
-    if (expert_products(m, l.gate_e, counts, ms->pack_x.data(), ms->g.data(), timed)) return 1;
-    if (expert_products(m, l.up_e, counts, ms->pack_x.data(), ms->u.data(), timed)) return 1;
-    for (size_t i = 0; i < pairs * ff; i++) {  // silu_inplace then the element-wise product, decode.rs:10244-10248
-        const float g = ms->g[i];
-        ms->g[i] = g / (1.f + std::exp(-g));
-        ms->g[i] *= ms->u[i];
+        for (uint32_t t : ms->buckets[e]) std::memcpy(packed + at++ * d, x + (size_t)t * d, d * sizeof(float));
+    if (on_device) {
+        if (expert_ffn_on_device(m, l, counts, pairs, ms, timed)) return 1;
+    } else {
+        ms->g.resize(pairs * ff);
+        ms->u.resize(pairs * ff);
+        if (expert_products(m, l.gate_e, counts, ms->pack_x.data(), ms->g.data(), timed)) return 1;
+        if (expert_products(m, l.up_e, counts, ms->pack_x.data(), ms->u.data(), timed)) return 1;
+        for (size_t i = 0; i < pairs * ff; i++) {  // silu_inplace then the element-wise product, decode.rs:10244-10248
+            const float g = ms->g[i];
+            ms->g[i] = g / (1.f + std::exp(-g));
+            ms->g[i] *= ms->u[i];
+        }
+        if (expert_products(m, l.down_e, counts, ms->g.data(), ms->y.data(), timed)) return 1;
     }
-    if (expert_products(m, l.down_e, counts, ms->g.data(), ms->y.data(), timed)) return 1;
     std::fill(ffn_out, ffn_out + n * d, 0.f);  // fit() zero-fills (decode.rs:1816-1819, 10381)
     at = 0;
     for (size_t e = 0; e < ne; e++) {
@@ -733,7 +835,7 @@ int moe_ffn(lnm_model *m, Layer &l, size_t n, const float *x, float *ffn_out, Mo
                     w = ms->sel_w[(size_t)t * k + j];
                     break;
                 }
-            const float *src = &ms->y[at++ * d];
+            const float *src = expert_y + at++ * d;
             float *dst = ffn_out + (size_t)t * d;
             const float scale = 1.f;  // no ffn_down_exps.scale tensor on this architecture (expert_part_scale)
             for (size_t i = 0; i < d; i++) dst[i] += src[i] * w * scale;
@@ -1199,8 +1301,8 @@ int lnm_moe_ffn(lnm_model *model, size_t layer, size_t n_tokens, const float *x,
     if (layer >= model->layers.size() || !model->layers[layer].moe) return fail("layer has no routed feed-forward");
     if (n_tokens == 0) return fail("empty batch");
     try {
-        MoeScratch ms;
-        return moe_ffn(model, model->layers[layer], n_tokens, x, ffn_out, &ms, nullptr);
+        if (!model->moe_entry) model->moe_entry = std::make_unique<MoeScratch>();  // kept: its device buffers are grow-only
+        return moe_ffn(model, model->layers[layer], n_tokens, x, ffn_out, model->moe_entry.get(), nullptr);
     } catch (const std::exception &e) {
         return fail(std::string("routed feed-forward: ") + e.what());
     }

@@ -172,7 +172,7 @@ def test_reference_session_scenario_on_every_path(pkg, llama, tmp_path, kind):
         assert got.argmax(axis=1).tolist() == want.argmax(axis=1).tolist(), key
 
 
-def test_mixtral_shaped_routed_layer_matches_the_cpu_path(pkg, llama, tmp_path):
+def test_mixtral_shaped_routed_layer_matches_the_cpu_path(pkg, llama, tmp_path, monkeypatch):
     """Benchmark configuration 5 as one checked result: 64 tokens, router logits of about unit deviation,
     softmax, top-2 of 8 experts, tokens grouped per expert, Q4_K gate / up (4096 -> 14336) and down
     (14336 -> 4096), weighted scatter-add - the whole layer on the GPU route against the same host code over
@@ -193,6 +193,16 @@ def test_mixtral_shaped_routed_layer_matches_the_cpu_path(pkg, llama, tmp_path):
     # one token alone takes the single-token kernels for its two experts: same row up to summation order
     alone = gpu.moe_ffn(0, x[5:6])
     assert np.all(np.abs(alone[0].astype(np.float64) - want[5]) <= 1e-4 * np.maximum(np.abs(want[5]), rms / 4))
+    # the projections are chained on the device (rows up once, SiLU * up there, down outputs back); with
+    # LLAMA_HIP_MOE_HOST_SWIGLU every projection is a call through host buffers and SiLU * up runs on the host, the
+    # reference's call structure: same products, exp of the host instead of the device's
+    monkeypatch.setenv("LLAMA_HIP_MOE_HOST_SWIGLU", "1")
+    through_host = gpu.moe_ffn(0, x)
+    monkeypatch.delenv("LLAMA_HIP_MOE_HOST_SWIGLU")
+    err = np.abs(through_host.astype(np.float64) - want)
+    assert np.all(err <= 1e-4 * np.maximum(np.abs(want), rms / 4))
+    assert np.abs(through_host.astype(np.float64) - got).max() <= 2e-5 * rms
+    assert np.array_equal(gpu.moe_ffn(0, x), got)  # and back: the same bits as before
 
 
 def test_config4_full_size_greedy_decode_on_every_path(pkg, llama, tmp_path):
