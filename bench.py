@@ -341,10 +341,11 @@ def other_workloads(pkg, hip, gpu, stream, rng, cpu):
     xd.free(); hd_.free(); gd.free(); ud.free(); yd2.free()
 
     # The same layer as the reference runs it, routing included (langtax/src/decode.rs:9938-10292): a Mixtral-shaped
-    # layer of a synthetic GGUF, 64 tokens through the host code - router product, softmax, top-2, grouping on the
-    # host, the packed rows to the device once, the three grouped expert products and SiLU * up chained there, the
-    # down outputs back, the weighted scatter on the host (LLAMA_HIP_MOE_HOST_SWIGLU=1: every projection a call
-    # through host buffers and SiLU * up on the host, as the reference's seam has it).
+    # layer of a synthetic GGUF, 64 tokens through the host code - the rows to the device once, the router product
+    # there, its logits back for softmax, top-2 and grouping on the host, the bucket order up, then gather, the three
+    # grouped expert products, SiLU * up and the weighted scatter chained on the device, the result back
+    # (LLAMA_HIP_MOE_HOST_SWIGLU=1: every product a call through host buffers, SiLU * up and the scatter on the
+    # host, as the reference's seam has it).
     import tempfile
     L = importlib.import_module("llama-rust_amd.llama")
     with tempfile.TemporaryDirectory() as tmp:
@@ -360,10 +361,11 @@ def other_workloads(pkg, hip, gpu, stream, rng, cpu):
             got = model.moe_ffn(0, xt)
         host_us = (time.perf_counter() - t0) / reps * 1e6
         entry = {"call_us": round(host_us, 1), "tokens": n_tok, "experts": n_exp, "top_k": 2,
-                 "scope": ("whole routed feed-forward, host routing and scatter: router product through the seam; "
-                           + ("gate, up, down as grouped calls through host buffers, SiLU*up on the host"
+                 "scope": ("whole routed feed-forward, host softmax / top-k / grouping: "
+                           + ("router, gate, up, down as calls through host buffers, SiLU*up and scatter on the host"
                               if os.environ.get("LLAMA_HIP_MOE_HOST_SWIGLU") else
-                              "one upload of the packed rows, gate / up / SiLU*up / down chained on the device, one download"))}
+                              "rows up once, router product, gather, gate / up / SiLU*up / down and scatter chained on the device, "
+                              "logits and the result back"))}
         if cpu:
             ref = L.Llama(path=path, products=L.CALLBACK,
                           matmul=lambda ty, n_rows, n_cols, n_tokens, w, x: O.gemm(ty, n_cols, n_tokens, w, x, n_rows, simd=True, threads=0))

@@ -343,19 +343,19 @@ struct MoeScratch {
     std::vector<float> logits, sel_w, pack_x, g, u, y;
     std::vector<uint32_t> sel_e, order;
     std::vector<std::vector<uint32_t>> buckets;
-    // Resident route: the packed rows go to the device once and gate, up, SiLU(gate) * up and down follow each
-    // other there (moe_ffn); grow-only buffers and a stream of the scratch's own.
-    float *d_x = nullptr, *d_g = nullptr, *d_u = nullptr, *d_y = nullptr;
-    float *h_x = nullptr, *h_y = nullptr;  // pinned: the packed rows and the down outputs on the host side of the copies
-    size_t cap_x = 0, cap_g = 0, cap_u = 0, cap_y = 0, cap_hx = 0, cap_hy = 0;  // floats
+    // Resident route (moe_ffn_on_device): grow-only device buffers, pinned staging and a stream of the scratch's own.
+    // io: the n x n_embd rows in and the result out; small: logits, bucket order, weights.
+    float *d_io = nullptr, *d_small = nullptr, *d_x = nullptr, *d_g = nullptr, *d_u = nullptr, *d_y = nullptr;
+    float *h_io = nullptr, *h_small = nullptr;
+    size_t cap_io = 0, cap_small = 0, cap_x = 0, cap_g = 0, cap_u = 0, cap_y = 0, cap_hio = 0, cap_hsmall = 0;  // floats
     hipStream_t stream = nullptr;
     MoeScratch() = default;
     MoeScratch(const MoeScratch &) = delete;
     MoeScratch &operator=(const MoeScratch &) = delete;
     ~MoeScratch() {
-        for (float *p : {d_x, d_g, d_u, d_y})
+        for (float *p : {d_io, d_small, d_x, d_g, d_u, d_y})
             if (p) (void)hipFree(p);
-        for (float *p : {h_x, h_y})
+        for (float *p : {h_io, h_small})
             if (p) (void)hipHostFree(p);
         if (stream) (void)hipStreamDestroy(stream);
     }
@@ -687,84 +687,32 @@ int expert_products(lnm_model *m, std::vector<Mat> &parts, const std::vector<siz
     return 0;
 }
 
-// The routed feed-forward of architecture llama with experts (Mixtral-shaped), langtax/src/decode.rs:10366-10409
-// (llama_moe_into: softmax over all experts, then top-k, weights renormalised with the 2^-14 clamp and applied
-// after the expert, SwiGLU, no shared expert), through softmax_routed_layer 9938-9966:
-//   route_softmax_tokens 9969-10004   router product, per token softmax -> topk -> router weights
-//   grouped_routed_ffn 10006-10060    token indices bucketed per expert, experts in ascending order
-//   grouped_one_expert 10062-10116    the bucket's rows packed contiguously
-//   swiglu_expert_gemm 10148-10261    gate and up products, SiLU(gate) * up, down product
-//   scatter_expert_rows 10263-10292   ffn_out[t] += y[i] * w(t, e)
-// x: n x n_embd rows (already normed), ffn_out: n x n_embd, overwritten.
 __global__ void dd_swiglu_kernel(float *gate, const float *up, uint32_t n);  // with the device session's kernels below
 
-// gate, up, SiLU(gate) * up and down of every non-empty expert with the packed rows uploaded once and nothing
-// but the down outputs coming back: three grouped launches and one element-wise kernel on one stream
-// (decode.rs:10148-10261 without its host round trips between the products).
-int expert_ffn_on_device(lnm_model *m, Layer &l, const std::vector<size_t> &counts, size_t pairs, MoeScratch *ms,
-                         lnm_session *timed) {
-    const auto t0 = wall_clock::now();
-    const size_t d = m->hp.n_embd, ff = l.gate_e[0].n_rows;
-    std::vector<const lnh_matrix *> hg, hu, hd;
-    std::vector<size_t> toks;
-    for (size_t e = 0; e < counts.size(); e++) {
-        if (counts[e] == 0) continue;
-        if (ensure_resident(m, l.gate_e[e]) != 0 || ensure_resident(m, l.up_e[e]) != 0 || ensure_resident(m, l.down_e[e]) != 0)
-            return 1;
-        hg.push_back(l.gate_e[e].resident);
-        hu.push_back(l.up_e[e].resident);
-        hd.push_back(l.down_e[e].resident);
-        toks.push_back(counts[e]);
-    }
-    if (pairs * ff > UINT32_MAX) return fail("routed feed-forward: too many expert rows for one call");
-    auto grow = [&](float **p, size_t *cap, size_t want) {
-        if (*cap >= want) return hipSuccess;
-        if (*p) (void)hipFree(*p);
-        *p = nullptr;
-        *cap = 0;
-        const hipError_t e = hipMalloc(reinterpret_cast<void **>(p), want * sizeof(float));
-        if (e == hipSuccess) *cap = want;
-        return e;
-    };
-    hipError_t e = ms->stream ? hipSuccess : hipStreamCreateWithFlags(&ms->stream, hipStreamNonBlocking);
-    if (e == hipSuccess) e = grow(&ms->d_x, &ms->cap_x, pairs * d);
-    if (e == hipSuccess) e = grow(&ms->d_g, &ms->cap_g, pairs * ff);
-    if (e == hipSuccess) e = grow(&ms->d_u, &ms->cap_u, pairs * ff);
-    if (e == hipSuccess) e = grow(&ms->d_y, &ms->cap_y, pairs * d);
-    if (e == hipSuccess) e = hipMemcpyAsync(ms->d_x, ms->h_x, pairs * d * sizeof(float), hipMemcpyHostToDevice, ms->stream);
-    if (e != hipSuccess) return fail(std::string("routed feed-forward: ") + hipGetErrorString(e));
-    if (lnh_gemm_grouped_device(m->exec, hg.size(), hg.data(), toks.data(), ms->d_x, ms->d_g, ms->stream) != 0 ||
-        lnh_gemm_grouped_device(m->exec, hu.size(), hu.data(), toks.data(), ms->d_x, ms->d_u, ms->stream) != 0)
-        return fail(std::string(lnh_last_error(m->exec)) + " (" + l.gate_e[0].name + ")");
-    const uint32_t n_h = (uint32_t)(pairs * ff);
-    hipLaunchKernelGGL(dd_swiglu_kernel, dim3((n_h + 1023) / 1024 < 4096 ? (n_h + 1023) / 1024 : 4096), dim3(256), 0, ms->stream,
-                       ms->d_g, ms->d_u, n_h);
-    e = hipGetLastError();
-    if (e != hipSuccess) return fail(std::string("routed feed-forward: ") + hipGetErrorString(e));
-    if (lnh_gemm_grouped_device(m->exec, hd.size(), hd.data(), toks.data(), ms->d_g, ms->d_y, ms->stream) != 0)
-        return fail(std::string(lnh_last_error(m->exec)) + " (" + l.down_e[0].name + ")");
-    e = hipMemcpyAsync(ms->h_y, ms->d_y, pairs * d * sizeof(float), hipMemcpyDeviceToHost, ms->stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(ms->stream);
-    if (e != hipSuccess) return fail(std::string("routed feed-forward: ") + hipGetErrorString(e));
-    if (timed) {
-        timed->products_s += since(t0);
-        timed->n_products += 3 * toks.size();
-    }
-    return 0;
+// packed[i] = x[row_of[i]]: the rows of every expert's bucket, contiguous (grouped_one_expert, decode.rs:10062-10116).
+__global__ __launch_bounds__(256) void moe_gather_kernel(const float *x, const uint32_t *row_of, uint32_t d, float *packed) {
+    const float4 *src = reinterpret_cast<const float4 *>(x + (size_t)row_of[blockIdx.x] * d);
+    float4 *dst = reinterpret_cast<float4 *>(packed + (size_t)blockIdx.x * d);
+    for (uint32_t i = threadIdx.x; i < d / 4; i += blockDim.x) dst[i] = src[i];
 }
 
-int moe_ffn(lnm_model *m, Layer &l, size_t n, const float *x, float *ffn_out, MoeScratch *ms, lnm_session *timed) {
-    const lnm_hparams &hp = m->hp;
-    const size_t d = hp.n_embd, ne = hp.n_expert, k = hp.n_expert_used, ff = l.gate_e[0].n_rows;
-    ms->logits.resize(n * ne);
-    {
-        const auto t0 = wall_clock::now();
-        if (product_routed(m, l.gate_inp, n, x, ms->logits.data()) != 0) return 1;
-        if (timed) {
-            timed->products_s += since(t0);
-            timed->n_products++;
-        }
+// out[t] = the token's expert outputs times their router weights, added in ascending expert order onto zero
+// (scatter_expert_rows, decode.rs:10263-10292: ffn_out[t] += y[i] * w over the experts in ascending order).
+// pair_of / w_of: per token its k selections in that order (row of y, weight).
+__global__ __launch_bounds__(256) void moe_scatter_kernel(const float *y, const uint32_t *pair_of, const float *w_of, uint32_t k,
+                                                          uint32_t d, float *out) {
+    const uint32_t t = blockIdx.x;
+    for (uint32_t i = threadIdx.x; i < d; i += blockDim.x) {
+        float o = 0.f;
+        for (uint32_t j = 0; j < k; j++) o += y[(size_t)pair_of[t * k + j] * d + i] * w_of[t * k + j];
+        out[(size_t)t * d + i] = o;
     }
+}
+
+// softmax -> topk -> router weights per token, tokens bucketed per expert (route_softmax_tokens 9969-10004,
+// grouped_routed_ffn 10006-10060); logits in ms->logits, overwritten by the probabilities.
+int moe_route(const lnm_hparams &hp, size_t n, MoeScratch *ms, std::vector<size_t> *counts, size_t *pairs) {
+    const size_t ne = hp.n_expert, k = hp.n_expert_used;
     ms->sel_e.resize(n * k);
     ms->sel_w.resize(n * k);
     for (size_t t = 0; t < n; t++) {
@@ -778,64 +726,171 @@ int moe_ffn(lnm_model *m, Layer &l, size_t n, const float *x, float *ffn_out, Mo
     for (auto &b : ms->buckets) b.clear();
     for (size_t t = 0; t < n; t++)
         for (size_t j = 0; j < k; j++) ms->buckets[ms->sel_e[t * k + j]].push_back((uint32_t)t);
-    std::vector<size_t> counts(ne);
-    size_t pairs = 0;
-    for (size_t e = 0; e < ne; e++) pairs += counts[e] = ms->buckets[e].size();
-    // LLAMA_HIP_MOE_HOST_SWIGLU set: every projection a grouped call of its own through host buffers, SiLU * up on
-    // the host, as the reference's seam does it
-    const bool host_swiglu = std::getenv("LLAMA_HIP_MOE_HOST_SWIGLU") != nullptr;  // read per call: tests switch it
-    const bool on_device = m->route == LNM_PRODUCTS_RESIDENT && !host_swiglu && pairs != 0;
-    float *packed = nullptr, *expert_y = nullptr;
-    if (on_device) {
-        auto grow_pinned = [](float **p, size_t *cap, size_t want) {
-            if (*cap >= want) return hipSuccess;
-            if (*p) (void)hipHostFree(*p);
-            *p = nullptr;
-            *cap = 0;
-            const hipError_t e = hipHostMalloc(reinterpret_cast<void **>(p), want * sizeof(float), hipHostMallocDefault);
-            if (e == hipSuccess) *cap = want;
-            return e;
-        };
-        hipError_t e = grow_pinned(&ms->h_x, &ms->cap_hx, pairs * d);
-        if (e == hipSuccess) e = grow_pinned(&ms->h_y, &ms->cap_hy, pairs * d);
-        if (e != hipSuccess) return fail(std::string("routed feed-forward: ") + hipGetErrorString(e));
-        packed = ms->h_x;
-        expert_y = ms->h_y;
-    } else {
-        ms->pack_x.resize(pairs * d);
-        ms->y.resize(pairs * d);
-        packed = ms->pack_x.data();
-        expert_y = ms->y.data();
+    counts->assign(ne, 0);
+    *pairs = 0;
+    for (size_t e = 0; e < ne; e++) *pairs += (*counts)[e] = ms->buckets[e].size();
+    return 0;
+}
+
+// token_expert_weight: the first selection of expert e by token t
+float moe_weight(const MoeScratch *ms, size_t k, uint32_t t, size_t e) {
+    for (size_t j = 0; j < k; j++)
+        if (ms->sel_e[(size_t)t * k + j] == e) return ms->sel_w[(size_t)t * k + j];
+    return 0.f;
+}
+
+// The routed feed-forward with the resident products chained on the device: the rows go up once (pinned staging),
+// the router product runs there and only its n x n_expert logits come back for the host's routing; then the
+// bucket order goes up (a few KB), the rows are gathered, gate and up are grouped launches, SiLU(gate) * up an
+// element-wise kernel, down a grouped launch, the scatter a kernel, and the n x n_embd result comes back: two host
+// synchronisations, no expert output ever on the host.  Same products and the same order of additions as moe_ffn's
+// host form; SiLU with the device's expf.
+int moe_ffn_on_device(lnm_model *m, Layer &l, size_t n, const float *x, float *ffn_out, MoeScratch *ms, lnm_session *timed) {
+    const lnm_hparams &hp = m->hp;
+    const size_t d = hp.n_embd, ne = hp.n_expert, k = hp.n_expert_used, ff = l.gate_e[0].n_rows;
+    const auto t0 = wall_clock::now();
+    auto grow = [](float **p, size_t *cap, size_t want, bool pinned) {
+        if (*cap >= want) return hipSuccess;
+        if (*p) (void)(pinned ? hipHostFree(*p) : hipFree(*p));
+        *p = nullptr;
+        *cap = 0;
+        const hipError_t e = pinned ? hipHostMalloc(reinterpret_cast<void **>(p), want * sizeof(float), hipHostMallocDefault)
+                                    : hipMalloc(reinterpret_cast<void **>(p), want * sizeof(float));
+        if (e == hipSuccess) *cap = want;
+        return e;
+    };
+    auto hip_fail = [](hipError_t e) { return fail(std::string("routed feed-forward: ") + hipGetErrorString(e)); };
+    const size_t pairs = n * k, n_idx = pairs + n * k;  // every token selects k distinct experts
+    if (pairs * ff > UINT32_MAX || n * d > UINT32_MAX) return fail("routed feed-forward: too many rows for one call");
+    hipError_t e = ms->stream ? hipSuccess : hipStreamCreateWithFlags(&ms->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = grow(&ms->h_io, &ms->cap_hio, n * d, true);
+    if (e == hipSuccess) e = grow(&ms->h_small, &ms->cap_hsmall, n * ne + n_idx + n * k, true);
+    if (e == hipSuccess) e = grow(&ms->d_io, &ms->cap_io, n * d, false);
+    if (e == hipSuccess) e = grow(&ms->d_small, &ms->cap_small, n * ne + n_idx + n * k, false);
+    if (e == hipSuccess) e = grow(&ms->d_x, &ms->cap_x, pairs * d, false);
+    if (e == hipSuccess) e = grow(&ms->d_g, &ms->cap_g, pairs * ff, false);
+    if (e == hipSuccess) e = grow(&ms->d_u, &ms->cap_u, pairs * ff, false);
+    if (e == hipSuccess) e = grow(&ms->d_y, &ms->cap_y, pairs * d, false);
+    if (e != hipSuccess) return hip_fail(e);
+    float *h_logits = ms->h_small, *d_logits = ms->d_small;
+    uint32_t *h_idx = reinterpret_cast<uint32_t *>(ms->h_small + n * ne), *d_idx = reinterpret_cast<uint32_t *>(ms->d_small + n * ne);
+    float *h_w = ms->h_small + n * ne + n_idx, *d_w = ms->d_small + n * ne + n_idx;
+
+    // rows up, router product, logits back
+    std::memcpy(ms->h_io, x, n * d * sizeof(float));
+    e = hipMemcpyAsync(ms->d_io, ms->h_io, n * d * sizeof(float), hipMemcpyHostToDevice, ms->stream);
+    if (e != hipSuccess) return hip_fail(e);
+    if (ensure_resident(m, l.gate_inp) != 0) return 1;
+    if (lnh_gemm_device(m->exec, l.gate_inp.resident, n, ms->d_io, d_logits, ms->stream) != 0)
+        return fail(std::string(lnh_last_error(m->exec)) + " (" + l.gate_inp.name + ")");
+    e = hipMemcpyAsync(h_logits, d_logits, n * ne * sizeof(float), hipMemcpyDeviceToHost, ms->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ms->stream);
+    if (e != hipSuccess) return hip_fail(e);
+    ms->logits.assign(h_logits, h_logits + n * ne);
+    std::vector<size_t> counts;
+    size_t routed = 0;
+    if (moe_route(hp, n, ms, &counts, &routed)) return 1;
+    if (routed != pairs) return fail("routed feed-forward: a token selected an expert twice");
+
+    // bucket order: the row of every packed position; per token its selections in ascending expert order
+    std::vector<uint32_t> filled(n, 0);
+    size_t at = 0;
+    for (size_t ex = 0; ex < ne; ex++)
+        for (uint32_t t : ms->buckets[ex]) {
+            h_idx[at] = t;
+            const size_t slot = (size_t)t * k + filled[t]++;
+            h_idx[pairs + slot] = (uint32_t)at;
+            h_w[slot] = moe_weight(ms, k, t, ex);
+            at++;
+        }
+    e = hipMemcpyAsync(d_idx, h_idx, (n_idx + n * k) * sizeof(float), hipMemcpyHostToDevice, ms->stream);  // indices and weights are adjacent
+    if (e != hipSuccess) return hip_fail(e);
+    std::vector<const lnh_matrix *> hg, hu, hdn;
+    std::vector<size_t> toks;
+    for (size_t ex = 0; ex < ne; ex++) {
+        if (counts[ex] == 0) continue;
+        if (ensure_resident(m, l.gate_e[ex]) != 0 || ensure_resident(m, l.up_e[ex]) != 0 || ensure_resident(m, l.down_e[ex]) != 0)
+            return 1;
+        hg.push_back(l.gate_e[ex].resident);
+        hu.push_back(l.up_e[ex].resident);
+        hdn.push_back(l.down_e[ex].resident);
+        toks.push_back(counts[ex]);
     }
+    hipLaunchKernelGGL(moe_gather_kernel, dim3((uint32_t)pairs), dim3(256), 0, ms->stream, ms->d_io, d_idx, (uint32_t)d, ms->d_x);
+    if ((e = hipGetLastError()) != hipSuccess) return hip_fail(e);
+    if (lnh_gemm_grouped_device(m->exec, hg.size(), hg.data(), toks.data(), ms->d_x, ms->d_g, ms->stream) != 0 ||
+        lnh_gemm_grouped_device(m->exec, hu.size(), hu.data(), toks.data(), ms->d_x, ms->d_u, ms->stream) != 0)
+        return fail(std::string(lnh_last_error(m->exec)) + " (" + l.gate_e[0].name + ")");
+    const uint32_t n_h = (uint32_t)(pairs * ff);
+    hipLaunchKernelGGL(dd_swiglu_kernel, dim3((n_h + 1023) / 1024 < 4096 ? (n_h + 1023) / 1024 : 4096), dim3(256), 0, ms->stream,
+                       ms->d_g, ms->d_u, n_h);
+    if ((e = hipGetLastError()) != hipSuccess) return hip_fail(e);
+    if (lnh_gemm_grouped_device(m->exec, hdn.size(), hdn.data(), toks.data(), ms->d_g, ms->d_y, ms->stream) != 0)
+        return fail(std::string(lnh_last_error(m->exec)) + " (" + l.down_e[0].name + ")");
+    hipLaunchKernelGGL(moe_scatter_kernel, dim3((uint32_t)n), dim3(256), 0, ms->stream, ms->d_y, d_idx + pairs, d_w, (uint32_t)k,
+                       (uint32_t)d, ms->d_io);
+    if ((e = hipGetLastError()) != hipSuccess) return hip_fail(e);
+    e = hipMemcpyAsync(ms->h_io, ms->d_io, n * d * sizeof(float), hipMemcpyDeviceToHost, ms->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ms->stream);
+    if (e != hipSuccess) return hip_fail(e);
+    std::memcpy(ffn_out, ms->h_io, n * d * sizeof(float));
+    if (timed) {
+        timed->products_s += since(t0);
+        timed->n_products += 1 + 3 * toks.size();
+    }
+    return 0;
+}
+
+// The routed feed-forward of architecture llama with experts (Mixtral-shaped), langtax/src/decode.rs:10366-10409
+// (llama_moe_into: softmax over all experts, then top-k, weights renormalised with the 2^-14 clamp and applied
+// after the expert, SwiGLU, no shared expert), through softmax_routed_layer 9938-9966:
+//   route_softmax_tokens 9969-10004   router product, per token softmax -> topk -> router weights
+//   grouped_routed_ffn 10006-10060    token indices bucketed per expert, experts in ascending order
+//   grouped_one_expert 10062-10116    the bucket's rows packed contiguously
+//   swiglu_expert_gemm 10148-10261    gate and up products, SiLU(gate) * up, down product
+//   scatter_expert_rows 10263-10292   ffn_out[t] += y[i] * w(t, e)
+// x: n x n_embd rows (already normed), ffn_out: n x n_embd, overwritten.
+// Resident route: moe_ffn_on_device, unless LLAMA_HIP_MOE_HOST_SWIGLU is set (then, as in the reference's seam, every
+// product is a call through host buffers and SiLU * up and the scatter run here).
+int moe_ffn(lnm_model *m, Layer &l, size_t n, const float *x, float *ffn_out, MoeScratch *ms, lnm_session *timed) {
+    const lnm_hparams &hp = m->hp;
+    const size_t d = hp.n_embd, ne = hp.n_expert, k = hp.n_expert_used, ff = l.gate_e[0].n_rows;
+    if (m->route == LNM_PRODUCTS_RESIDENT && std::getenv("LLAMA_HIP_MOE_HOST_SWIGLU") == nullptr)  // read per call: tests switch it
+        return moe_ffn_on_device(m, l, n, x, ffn_out, ms, timed);
+    ms->logits.resize(n * ne);
+    {
+        const auto t0 = wall_clock::now();
+        if (product_routed(m, l.gate_inp, n, x, ms->logits.data()) != 0) return 1;
+        if (timed) {
+            timed->products_s += since(t0);
+            timed->n_products++;
+        }
+    }
+    std::vector<size_t> counts;
+    size_t pairs = 0;
+    if (moe_route(hp, n, ms, &counts, &pairs)) return 1;
     // every expert's rows, expert after expert in ascending order
+    ms->pack_x.resize(pairs * d);
+    ms->g.resize(pairs * ff);
+    ms->u.resize(pairs * ff);
+    ms->y.resize(pairs * d);
     size_t at = 0;
     for (size_t e = 0; e < ne; e++)
-        for (uint32_t t : ms->buckets[e]) std::memcpy(packed + at++ * d, x + (size_t)t * d, d * sizeof(float));
-    if (on_device) {
-        if (expert_ffn_on_device(m, l, counts, pairs, ms, timed)) return 1;
-    } else {
-        ms->g.resize(pairs * ff);
-        ms->u.resize(pairs * ff);
-        if (expert_products(m, l.gate_e, counts, ms->pack_x.data(), ms->g.data(), timed)) return 1;
-        if (expert_products(m, l.up_e, counts, ms->pack_x.data(), ms->u.data(), timed)) return 1;
-        for (size_t i = 0; i < pairs * ff; i++) {  // silu_inplace then the element-wise product, decode.rs:10244-10248
-            const float g = ms->g[i];
-            ms->g[i] = g / (1.f + std::exp(-g));
-            ms->g[i] *= ms->u[i];
-        }
-        if (expert_products(m, l.down_e, counts, ms->g.data(), ms->y.data(), timed)) return 1;
+        for (uint32_t t : ms->buckets[e]) std::memcpy(&ms->pack_x[at++ * d], x + (size_t)t * d, d * sizeof(float));
+    if (expert_products(m, l.gate_e, counts, ms->pack_x.data(), ms->g.data(), timed)) return 1;
+    if (expert_products(m, l.up_e, counts, ms->pack_x.data(), ms->u.data(), timed)) return 1;
+    for (size_t i = 0; i < pairs * ff; i++) {  // silu_inplace then the element-wise product, decode.rs:10244-10248
+        const float g = ms->g[i];
+        ms->g[i] = g / (1.f + std::exp(-g));
+        ms->g[i] *= ms->u[i];
     }
+    if (expert_products(m, l.down_e, counts, ms->g.data(), ms->y.data(), timed)) return 1;
     std::fill(ffn_out, ffn_out + n * d, 0.f);  // fit() zero-fills (decode.rs:1816-1819, 10381)
     at = 0;
     for (size_t e = 0; e < ne; e++) {
         for (uint32_t t : ms->buckets[e]) {
-            float w = 0.f;  // token_expert_weight: the first selection of this expert by the token
-            for (size_t j = 0; j < k; j++)
-                if (ms->sel_e[(size_t)t * k + j] == e) {
-                    w = ms->sel_w[(size_t)t * k + j];
-                    break;
-                }
-            const float *src = expert_y + at++ * d;
+            const float w = moe_weight(ms, k, t, e);
+            const float *src = &ms->y[at++ * d];
             float *dst = ffn_out + (size_t)t * d;
             const float scale = 1.f;  // no ffn_down_exps.scale tensor on this architecture (expert_part_scale)
             for (size_t i = 0; i < d; i++) dst[i] += src[i] * w * scale;
