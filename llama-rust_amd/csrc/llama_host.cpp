@@ -701,12 +701,19 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(const float *x, const u
 // pair_of / w_of: per token its k selections in that order (row of y, weight).
 __global__ __launch_bounds__(256) void moe_scatter_kernel(const float *y, const uint32_t *pair_of, const float *w_of, uint32_t k,
                                                           uint32_t d, float *out) {
-    const uint32_t t = blockIdx.x;
-    for (uint32_t i = threadIdx.x; i < d; i += blockDim.x) {
-        float o = 0.f;
-        for (uint32_t j = 0; j < k; j++) o += y[(size_t)pair_of[t * k + j] * d + i] * w_of[t * k + j];
-        out[(size_t)t * d + i] = o;
+    const uint32_t t = blockIdx.x;  // blockIdx.y: which 1024 columns (four per thread; d is a multiple of 4)
+    const uint32_t i = (blockIdx.y * blockDim.x + threadIdx.x) * 4;
+    if (i >= d) return;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t j = 0; j < k; j++) {
+        const float4 v = *reinterpret_cast<const float4 *>(y + (size_t)pair_of[t * k + j] * d + i);
+        const float w = w_of[t * k + j];
+        o.x += v.x * w;
+        o.y += v.y * w;
+        o.z += v.z * w;
+        o.w += v.w * w;
     }
+    *reinterpret_cast<float4 *>(out + (size_t)t * d + i) = o;
 }
 
 // softmax -> topk -> router weights per token, tokens bucketed per expert (route_softmax_tokens 9969-10004,
@@ -827,8 +834,8 @@ int moe_ffn_on_device(lnm_model *m, Layer &l, size_t n, const float *x, float *f
     if ((e = hipGetLastError()) != hipSuccess) return hip_fail(e);
     if (lnh_gemm_grouped_device(m->exec, hdn.size(), hdn.data(), toks.data(), ms->d_g, ms->d_y, ms->stream) != 0)
         return fail(std::string(lnh_last_error(m->exec)) + " (" + l.down_e[0].name + ")");
-    hipLaunchKernelGGL(moe_scatter_kernel, dim3((uint32_t)n), dim3(256), 0, ms->stream, ms->d_y, d_idx + pairs, d_w, (uint32_t)k,
-                       (uint32_t)d, ms->d_io);
+    hipLaunchKernelGGL(moe_scatter_kernel, dim3((uint32_t)n, (uint32_t)((d + 1023) / 1024)), dim3(256), 0, ms->stream, ms->d_y,
+                       d_idx + pairs, d_w, (uint32_t)k, (uint32_t)d, ms->d_io);
     if ((e = hipGetLastError()) != hipSuccess) return hip_fail(e);
     e = hipMemcpyAsync(ms->h_io, ms->d_io, n * d * sizeof(float), hipMemcpyDeviceToHost, ms->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ms->stream);
@@ -855,7 +862,8 @@ int moe_ffn_on_device(lnm_model *m, Layer &l, size_t n, const float *x, float *f
 int moe_ffn(lnm_model *m, Layer &l, size_t n, const float *x, float *ffn_out, MoeScratch *ms, lnm_session *timed) {
     const lnm_hparams &hp = m->hp;
     const size_t d = hp.n_embd, ne = hp.n_expert, k = hp.n_expert_used, ff = l.gate_e[0].n_rows;
-    if (m->route == LNM_PRODUCTS_RESIDENT && std::getenv("LLAMA_HIP_MOE_HOST_SWIGLU") == nullptr)  // read per call: tests switch it
+    // (rows of whole float4: the gather and scatter kernels move them that way; the variable is read per call, tests switch it)
+    if (m->route == LNM_PRODUCTS_RESIDENT && d % 4 == 0 && std::getenv("LLAMA_HIP_MOE_HOST_SWIGLU") == nullptr)
         return moe_ffn_on_device(m, l, n, x, ffn_out, ms, timed);
     ms->logits.resize(n * ne);
     {
