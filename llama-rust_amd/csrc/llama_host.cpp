@@ -825,9 +825,31 @@ int moe_ffn_on_device(lnm_model *m, Layer &l, size_t n, const float *x, float *f
     }
     hipLaunchKernelGGL(moe_gather_kernel, dim3((uint32_t)pairs), dim3(256), 0, ms->stream, ms->d_io, d_idx, (uint32_t)d, ms->d_x);
     if ((e = hipGetLastError()) != hipSuccess) return hip_fail(e);
-    if (lnh_gemm_grouped_device(m->exec, hg.size(), hg.data(), toks.data(), ms->d_x, ms->d_g, ms->stream) != 0 ||
-        lnh_gemm_grouped_device(m->exec, hu.size(), hu.data(), toks.data(), ms->d_x, ms->d_u, ms->stream) != 0)
-        return fail(std::string(lnh_last_error(m->exec)) + " (" + l.gate_e[0].name + ")");
+    {
+        // gate and up of every expert as one batch: the experts of at most 16 rows first, then the others, so that
+        // products of one tile size lie together and share launches (up to eight each) - with eight products a
+        // launch has enough tiles to fill the chip without sharing columns, and no launch sums shares
+        std::vector<const lnh_matrix *> mats;
+        std::vector<size_t> rows;
+        std::vector<const float *> xs;
+        std::vector<float *> ys;
+        for (int big = 0; big < 2; big++) {
+            size_t at_x = 0, at_h = 0;
+            for (size_t i = 0; i < toks.size(); i++) {
+                if ((toks[i] > 16) == (big == 1))
+                    for (int up = 0; up < 2; up++) {
+                        mats.push_back(up ? hu[i] : hg[i]);
+                        rows.push_back(toks[i]);
+                        xs.push_back(ms->d_x + at_x);
+                        ys.push_back((up ? ms->d_u : ms->d_g) + at_h);
+                    }
+                at_x += toks[i] * d;
+                at_h += toks[i] * ff;
+            }
+        }
+        if (lnh_gemm_batch_device(m->exec, mats.size(), mats.data(), rows.data(), xs.data(), ys.data(), ms->stream) != 0)
+            return fail(std::string(lnh_last_error(m->exec)) + " (" + l.gate_e[0].name + ")");
+    }
     const uint32_t n_h = (uint32_t)(pairs * ff);
     hipLaunchKernelGGL(dd_swiglu_kernel, dim3((n_h + 1023) / 1024 < 4096 ? (n_h + 1023) / 1024 : 4096), dim3(256), 0, ms->stream,
                        ms->d_g, ms->d_u, n_h);
