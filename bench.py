@@ -334,6 +334,33 @@ def other_workloads(pkg, hip, gpu, stream, rng, cpu):
         "call_us": round(us, 2), "calls": 3, "tokens_per_expert": counts, "weight_gbs": round(wbytes / us / 1e3, 1),
         "frac": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4), "tflops": round(2.0 * pairs * 3 * FF * D / us / 1e6, 1),
         "bound": "hbm"}
+    # the same products with gate and up of all experts as ONE batch call (lnh_gemm_batch_device), the experts of
+    # at most 16 tokens first: eight products of one tile size per launch, no shared columns, no launch that sums
+    # shares - how the library's own routed layer issues them
+    def batches(i):
+        mats, toks, xs, ys = [], [], [], []
+        for big in (False, True):
+            ox = oh = 0
+            for e in range(n_exp):
+                if counts[e] and (counts[e] > 16) == big:
+                    for mset, out_buf in ((mg[i], gd), (mu[i], ud)):
+                        mats.append(mset[e]); toks.append(counts[e]); xs.append(xd.ptr + ox * 4); ys.append(out_buf.ptr + oh * 4)
+                ox += counts[e] * D
+                oh += counts[e] * FF
+        return gpu.make_batch(mats, toks, xs, ys)
+
+    pre = [batches(i) for i in range(sets)]
+
+    def layer_batched(i):
+        gpu.gemm_batch_device(pre[i], stream.ptr)
+        gpu.gemm_grouped_device(md[i], counts, hd_.ptr, yd2.ptr, stream.ptr)
+
+    g_ref = gd.to_numpy(np.float32).copy()
+    us_b = timed_us(hip, stream, layer_batched, sets, 5)
+    layer_batched(0); stream.synchronize()
+    if not np.allclose(gd.to_numpy(np.float32), g_ref, rtol=1e-4, atol=1e-4 * float(np.sqrt(np.mean(g_ref.astype(np.float64) ** 2)))):
+        raise RuntimeError("MoE layer: the batched gate/up products disagree with the grouped call's")
+    out["moe_layer_q4_k_8_experts_top2_64_tokens"]["call_us_gate_up_as_one_batch"] = round(us_b, 2)
     for group in (mg, mu, md):
         for ms_ in group:
             for m in ms_:
