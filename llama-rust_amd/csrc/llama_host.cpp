@@ -25,6 +25,7 @@
 #include <string>
 #include <thread>
 #include <map>
+#include <tuple>
 #include <vector>
 
 #include <hip/hip_runtime.h>
@@ -219,16 +220,23 @@ uint32_t argmax(const float *x, size_t n) {  // first maximum wins; langtax/src/
 }
 
 // Indices of the k largest values, descending, ties to the lower index (langtax/src/decode.rs:11363-11379:
-// ggml_argsort_top_k; a NaN compares as a tie).  False when k is 0 or exceeds n.
+// ggml_argsort_top_k).  The reference's comparator treats a NaN as a tie with everything, which is no order
+// at all once a NaN is present; here the order is total, as std::sort requires: numbers descending, then the
+// NaNs, equal keys by ascending index.  On inputs without NaN both give the same result.  False when k is 0 or
+// exceeds n.
 bool topk(const float *v, size_t n, size_t k, std::vector<uint32_t> *order) {
     if (k == 0 || k > n) return false;
     order->resize(n);
     for (size_t i = 0; i < n; i++) (*order)[i] = (uint32_t)i;
     std::sort(order->begin(), order->end(), [&](uint32_t a, uint32_t b) {
         const float va = v[a], vb = v[b];
-        if (vb < va) return true;    // a first: larger value
-        if (vb > va) return false;
-        return a < b;                // equal or unordered: lower index first
+        const bool na = va != va, nb = vb != vb;
+        if (na != nb) return nb;     // a number before a NaN
+        if (!na) {
+            if (vb < va) return true;    // a first: larger value
+            if (vb > va) return false;
+        }
+        return a < b;                // equal numbers, or two NaNs: lower index first
     });
     order->resize(k);
     return true;
@@ -783,6 +791,16 @@ int moe_ffn_on_device(lnm_model *m, Layer &l, size_t n, const float *x, float *f
     uint32_t *h_idx = reinterpret_cast<uint32_t *>(ms->h_small + n * ne), *d_idx = reinterpret_cast<uint32_t *>(ms->d_small + n * ne);
     float *h_w = ms->h_small + n * ne + n_idx, *d_w = ms->d_small + n * ne + n_idx;
 
+    // From the first enqueue on, every return that is not the normal one leaves work on the stream that still
+    // reads the pinned and device buffers: it waits for the stream before it hands them back to the next call
+    // (which copies into them and may free them to grow).
+    struct DrainOnError {
+        hipStream_t s;
+        bool armed;
+        ~DrainOnError() {
+            if (armed) (void)hipStreamSynchronize(s);
+        }
+    } drain{ms->stream, true};
     // rows up, router product, logits back
     std::memcpy(ms->h_io, x, n * d * sizeof(float));
     e = hipMemcpyAsync(ms->d_io, ms->h_io, n * d * sizeof(float), hipMemcpyHostToDevice, ms->stream);
@@ -797,19 +815,23 @@ int moe_ffn_on_device(lnm_model *m, Layer &l, size_t n, const float *x, float *f
     std::vector<size_t> counts;
     size_t routed = 0;
     if (moe_route(hp, n, ms, &counts, &routed)) return 1;
-    if (routed != pairs) return fail("routed feed-forward: a token selected an expert twice");
+    if (routed != pairs) return fail("routed feed-forward: the buckets do not hold k selections per token");
 
     // bucket order: the row of every packed position; per token its selections in ascending expert order
     std::vector<uint32_t> filled(n, 0);
     size_t at = 0;
-    for (size_t ex = 0; ex < ne; ex++)
+    for (size_t ex = 0; ex < ne; ex++) {
+        uint32_t before = UINT32_MAX;  // tokens ascend inside a bucket: a token twice in one would be adjacent
         for (uint32_t t : ms->buckets[ex]) {
+            if (t == before || t >= n || filled[t] >= k) return fail("routed feed-forward: a token selected an expert twice");
+            before = t;
             h_idx[at] = t;
             const size_t slot = (size_t)t * k + filled[t]++;
             h_idx[pairs + slot] = (uint32_t)at;
             h_w[slot] = moe_weight(ms, k, t, ex);
             at++;
         }
+    }
     e = hipMemcpyAsync(d_idx, h_idx, (n_idx + n * k) * sizeof(float), hipMemcpyHostToDevice, ms->stream);  // indices and weights are adjacent
     if (e != hipSuccess) return hip_fail(e);
     std::vector<const lnh_matrix *> hg, hu, hdn;
@@ -862,6 +884,7 @@ int moe_ffn_on_device(lnm_model *m, Layer &l, size_t n, const float *x, float *f
     e = hipMemcpyAsync(ms->h_io, ms->d_io, n * d * sizeof(float), hipMemcpyDeviceToHost, ms->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ms->stream);
     if (e != hipSuccess) return hip_fail(e);
+    drain.armed = false;  // the stream is idle
     std::memcpy(ffn_out, ms->h_io, n * d * sizeof(float));
     if (timed) {
         timed->products_s += since(t0);

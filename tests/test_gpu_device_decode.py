@@ -306,6 +306,28 @@ def test_split_activation_chain_and_separate_launches_give_the_same_session(pkg,
     assert logits_chained.view(np.uint32).tolist() == logits_separate.view(np.uint32).tolist()
 
 
+@pytest.mark.parametrize("block_type,n_seq,n_prompt", [(12, 3, 4), (12, 8, 18), (2, 32, 33), (8, 5, 30)])
+def test_split_activation_chain_where_n_ff_equals_n_embd(pkg, llama, tmp_path, monkeypatch, block_type, n_seq, n_prompt):
+    """n_ff == n_embd with one block dtype: the input of the down product and the input of the next layer's q, k, v
+    have the same dtype and column count, and must still be two buffers (the down product reads the one while its
+    epilogue writes the other).  Steps of 3..32 rows and prompt chunks of 3..32 tokens, chained and with
+    LLAMA_HIP_BATCH_UNFUSED: same tokens, same logits bit for bit."""
+    path = tmp_path / "square.gguf"
+    llama.write_synthetic_llama(path, n_layer=3, n_embd=512, n_head=8, n_head_kv=2, n_ff=512, n_vocab=2048,
+                                block_type=block_type, embd_type=block_type, output_type=block_type, seed=53)
+    m = llama.Llama(path=path)
+    rng = np.random.default_rng(11 + n_seq)
+    prompts = [rng.integers(0, 2048, int(n)).tolist() for n in rng.integers(1, 40, n_seq)]
+    chunk_prompt = rng.integers(0, 2048, n_prompt).tolist()
+    chained = m.batch_session(n_seq, 64).generate_greedy(prompts, 10)[0]
+    logits_chained = m.session(device_positions=64).forward(chunk_prompt)
+    monkeypatch.setenv("LLAMA_HIP_BATCH_UNFUSED", "1")
+    separate = m.batch_session(n_seq, 64).generate_greedy(prompts, 10)[0]
+    logits_separate = m.session(device_positions=64).forward(chunk_prompt)
+    assert chained.tolist() == separate.tolist()
+    assert logits_chained.view(np.uint32).tolist() == logits_separate.view(np.uint32).tolist()
+
+
 def test_batch_session_refuses_what_it_cannot_do(pkg, llama, tmp_path):
     path = tmp_path / "small.gguf"
     llama.write_synthetic_llama(path, n_layer=2, n_embd=256, n_head=4, n_head_kv=2, n_ff=512, n_vocab=512, seed=43)

@@ -478,9 +478,10 @@ def test_adversarial_activations_keep_the_reference_bound(pkg, gpu, ty):
 
 
 @pytest.mark.parametrize("ty", [K.Q4_0, K.Q5_0, K.Q5_1, K.Q8_0, K.Q4_K, K.Q6_K], ids=lambda t: O.TYPE_NAMES[t])
-def test_every_f16_scale_pattern_and_zero_blocks(pkg, gpu, ty):
-    """langtax/src/simd/tests.rs:795-828, 1481-1520: every finite binary16 pattern as a block
-    scale (subnormals must survive the hardware conversion), and all-zero blocks."""
+def test_zero_blocks_among_swept_f16_scales(pkg, gpu, ty):
+    """langtax/src/simd/tests.rs:1481-1520: all-zero blocks (scale bits and codes zero) among blocks whose scales walk
+    through every fifth finite binary16 pattern.  The whole sweep of langtax/src/simd/tests.rs:795-828, every pattern
+    through every kernel family, is test_gpu_sweeps.py::test_every_finite_f16_scale_pattern_through_every_kernel_family."""
     rng = np.random.default_rng(7)
     bits = np.array([b for b in range(0, 65536, 5) if (b >> 10) & 0x1f != 31], np.uint16)
     per_row = 4096 // K.QK[ty]
