@@ -355,11 +355,16 @@ def other_workloads(pkg, hip, gpu, stream, rng, cpu):
         gpu.gemm_batch_device(pre[i], stream.ptr)
         gpu.gemm_grouped_device(md[i], counts, hd_.ptr, yd2.ptr, stream.ptr)
 
-    g_ref = gd.to_numpy(np.float32).copy()
+    # what the three grouped calls of layer(0) left, against what the batched layer leaves in the same buffers
+    refs = {"gate": (gd, gd.to_numpy(np.float32).copy()), "up": (ud, ud.to_numpy(np.float32).copy()),
+            "down": (yd2, yd2.to_numpy(np.float32).copy())}
     us_b = timed_us(hip, stream, layer_batched, sets, 5)
+    for buf, _ in refs.values():
+        buf.fill_byte(0xff)   # NaN patterns: a job that wrote to the wrong place leaves them standing
     layer_batched(0); stream.synchronize()
-    if not np.allclose(gd.to_numpy(np.float32), g_ref, rtol=1e-4, atol=1e-4 * float(np.sqrt(np.mean(g_ref.astype(np.float64) ** 2)))):
-        raise RuntimeError("MoE layer: the batched gate/up products disagree with the grouped call's")
+    for name, (buf, ref) in refs.items():
+        if not np.allclose(buf.to_numpy(np.float32), ref, rtol=1e-4, atol=1e-4 * float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))):
+            raise RuntimeError(f"MoE layer: the batched layer's {name} products disagree with the grouped call's")
     out["moe_layer_q4_k_8_experts_top2_64_tokens"]["call_us_gate_up_as_one_batch"] = round(us_b, 2)
     for group in (mg, mu, md):
         for ms_ in group:

@@ -262,6 +262,12 @@ int lnh_validate(const float *actual, size_t actual_len, const double *expected,
 /* Packed bytes of one row, 0 if cols is not a whole number of blocks or the type is unknown
  * (langtax/src/quant.rs:4210-4218, 4254-4284, 5647-5682). */
 size_t lnh_row_bytes(uint32_t ggml_type, size_t cols);
+/* Device bytes a packed rows x cols matrix holds once it has met products of up to `tokens` tokens: the
+ * single-token layout, plus the multi-token layout when such a product reads it (tokens >= 3, quantized
+ * dtypes).  What a residency cache charges before the upload, where the reference charges rows * cols * 4
+ * (langtax/src/native_gpu.rs:178-182); after the product lnh_matrix_info gives the figure as it stands.
+ * 0 for an unknown dtype, columns that are not whole blocks, or a size beyond size_t. */
+size_t lnh_resident_bytes(uint32_t ggml_type, size_t rows, size_t cols, size_t tokens);
 
 /* ------------------------------------------------------------------ dispatch + residency
  * The layer above the executor: the twin of langtax/src/native_gpu.rs plus the

@@ -117,6 +117,7 @@ def load_library():
         "lnh_shape_checked": (C.c_int, [sz, sz, sz, sz, C.POINTER(u32), C.POINTER(u32)]),
         "lnh_validate": (C.c_int, [vp, sz, vp, sz]),
         "lnh_row_bytes": (sz, [u32, sz]),
+        "lnh_resident_bytes": (sz, [u32, sz, sz, sz]),
         "lnq_gemv": (C.c_int, [u32, sz, vp, sz, vp, sz, vp, sz]),
         "lnq_gemm": (C.c_int, [u32, sz, sz, vp, sz, vp, sz, vp, sz]),
         "lnq_gemm_grouped": (C.c_int, [u32, sz, sz, sz, pvp, sz, psz, vp, sz, vp, sz]),
@@ -215,6 +216,12 @@ def validate(actual, expected):
 
 def row_bytes(ggml_type, cols):
     return load_library().lnh_row_bytes(ggml_type, cols)
+
+
+def resident_bytes(ggml_type, rows, cols, tokens=1):
+    """Device bytes a packed rows x cols matrix holds once it has met products of up to `tokens` tokens
+    (0: no such matrix); what the residency layer charges before an upload."""
+    return load_library().lnh_resident_bytes(ggml_type, rows, cols, tokens)
 
 
 # ------------------------------------------------------------------ gpu.rs mirror

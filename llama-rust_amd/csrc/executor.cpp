@@ -1010,4 +1010,13 @@ int lnh_validate(const float *actual, size_t actual_len, const double *expected,
 
 size_t lnh_row_bytes(uint32_t type, size_t cols) { return nh::gguf_row_bytes(type, cols); }
 
+size_t lnh_resident_bytes(uint32_t type, size_t rows, size_t cols, size_t tokens) {
+    const size_t rb = nh::gguf_row_bytes(type, cols);
+    if (rb == 0 || rows == 0 || rows > UINT32_MAX || cols > UINT32_MAX || rb > SIZE_MAX / 4 / rows) return 0;
+    size_t bytes = nh::plane_spec(type, rows, cols).total;
+    if (nh::product_reads_tiled(type, tokens > UINT32_MAX ? UINT32_MAX : (uint32_t)tokens))
+        bytes += nh::tiled_spec(type, rows, cols).total;
+    return bytes;
+}
+
 }  // extern "C"

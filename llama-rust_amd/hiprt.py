@@ -65,6 +65,12 @@ class DeviceBuffer:
         check(rt().hipMemcpy(b.ptr, a.ctypes.data, a.nbytes, H2D), "hipMemcpy H2D")
         return b
 
+    def upload(self, a):
+        """Overwrite the start of the buffer with the bytes of `a` (synchronous)."""
+        a = np.ascontiguousarray(a)
+        assert a.nbytes <= self.nbytes
+        check(rt().hipMemcpy(self.ptr, a.ctypes.data, a.nbytes, H2D), "hipMemcpy H2D")
+
     def to_numpy(self, dtype, count=None):
         dt = np.dtype(dtype)
         n = self.nbytes // dt.itemsize if count is None else count

@@ -13,6 +13,17 @@ fn text(p: *const c_char) -> String {
     unsafe { CStr::from_ptr(p) }.to_string_lossy().into_owned()
 }
 
+/// Device bytes a packed `rows x cols` matrix holds once it has met products of up to `tokens` tokens
+/// (the single-token layout, plus the multi-token layout when such a product reads it): what a residency
+/// cache charges before the upload.  `None` for a dtype or shape the packed kernels do not take.
+pub fn resident_bytes(ggml_type: u32, rows: usize, cols: usize, tokens: usize) -> Option<usize> {
+    // SAFETY: a pure function of its arguments.
+    match unsafe { ffi::lnh_resident_bytes(ggml_type, rows, cols, tokens) } {
+        0 => None,
+        n => Some(n),
+    }
+}
+
 /// Immutable matrix uploaded once and retained on the GPU (stands in for `CudaMatrix`).  Packed
 /// uploads keep the GGUF bytes packed; `shape` is the logical rows x cols either way.
 pub struct HipMatrix {
@@ -96,13 +107,14 @@ impl HipGemv {
     /// Upload the GGUF bytes of a rows x cols tensor and keep them packed on the device.  Replaces
     /// `expand()` + `upload` in `langtax/src/native_gpu.rs:190-194`.
     pub fn upload_packed(&mut self, ggml_type: u32, rows: usize, cols: usize, packed: &[u8]) -> Result<HipMatrix, String> {
-        let mut raw = std::ptr::null_mut();
-        // SAFETY: `packed` is valid for `packed.len()` bytes during the synchronous call.
-        self.check(unsafe { ffi::lnh_upload_packed(self.raw, ggml_type, rows, cols, packed.as_ptr(), packed.len(), &mut raw) })?;
+        // the shape first: nothing can fail between the upload and the handle's owner
         let shape = Shape {
             rows: u32::try_from(rows).map_err(|_| "GEMV rows exceed u32")?,
             cols: u32::try_from(cols).map_err(|_| "GEMV columns exceed u32")?,
         };
+        let mut raw = std::ptr::null_mut();
+        // SAFETY: `packed` is valid for `packed.len()` bytes during the synchronous call.
+        self.check(unsafe { ffi::lnh_upload_packed(self.raw, ggml_type, rows, cols, packed.as_ptr(), packed.len(), &mut raw) })?;
         Ok(HipMatrix { raw, shape })
     }
 

@@ -7,8 +7,9 @@
 //! `gemm_grouped` issues the per-expert products of one MoE projection as one call.
 //!
 //! This crate is written against the C header and checked against it by
-//! `tests/test_rust_binding.py`; the image it was written in has no Rust toolchain, so it has
-//! not been compiled.
+//! `tests/test_rust_binding.py` (every `extern "C"` declaration against the header's, textually); the
+//! image it was written in has no Rust toolchain, so it has been neither compiled nor run: nothing
+//! beyond that signature check pins its behaviour.
 
 #[cfg(feature = "hip")]
 mod ffi {
@@ -62,6 +63,7 @@ mod ffi {
         pub fn lnh_shape_checked(rows: usize, cols: usize, weights_len: usize, input_len: usize, rows_out: *mut u32, cols_out: *mut u32) -> c_int;
         pub fn lnh_validate(actual: *const f32, actual_len: usize, expected: *const f64, expected_len: usize) -> c_int;
         pub fn lnh_row_bytes(ggml_type: u32, cols: usize) -> usize;
+        pub fn lnh_resident_bytes(ggml_type: u32, rows: usize, cols: usize, tokens: usize) -> usize;
         pub fn lnq_gemv(ggml_type: u32, n_cols: usize, w: *const u8, w_len: usize, x: *const f32, x_len: usize, y: *mut f32, y_len: usize) -> c_int;
         pub fn lnq_gemm(ggml_type: u32, n_cols: usize, n_tokens: usize, w: *const u8, w_len: usize, x: *const f32, x_len: usize, y: *mut f32, y_len: usize) -> c_int;
         pub fn lnq_gemm_grouped(ggml_type: u32, n_cols: usize, n_rows: usize, n_groups: usize, parts: *const *const u8, part_len: usize, tokens: *const usize, x: *const f32, x_len: usize, y: *mut f32, y_len: usize) -> c_int;
@@ -72,7 +74,7 @@ mod ffi {
 #[cfg(feature = "hip")]
 mod gpu;
 #[cfg(feature = "hip")]
-pub use gpu::{HipGemv, HipMatrix};
+pub use gpu::{HipGemv, HipMatrix, resident_bytes};
 
 /// ggml type ids of the eight dtypes the kernels handle (`langtax/src/gguf.rs:245-258`,
 /// `include/native_hip.h`).

@@ -64,6 +64,29 @@ def test_row_bytes(pkg):
     assert pkg.row_bytes(3, 256) == 0  # Q4_1 is outside the eight dtypes
 
 
+def test_resident_bytes_is_the_packed_size_once_or_about_twice(pkg):
+    """What a residency cache charges before an upload: every dtype holds its GGUF bytes once (plus plane alignment
+    and row padding) while it only meets one or two tokens; a quantized matrix that meets three or more holds the
+    second layout as well, F32 / F16 never do.  Nothing for shapes the packed kernels do not take."""
+    for ty in pkg.ALL_TYPES:
+        for rows, cols in ((4096, 4096), (1000, 14336), (3, 256)):
+            packed = rows * K.row_bytes(ty, cols)
+            one = pkg.resident_bytes(ty, rows, cols, 1)
+            assert one == pkg.resident_bytes(ty, rows, cols, 2)
+            assert packed <= one <= packed + 4 * (256 + 64) + 16 * rows
+            many = pkg.resident_bytes(ty, rows, cols, 3)
+            assert many == pkg.resident_bytes(ty, rows, cols, 512)
+            if ty in (pkg.F32, pkg.F16):
+                assert many == one
+            else:
+                tiled_rows = (rows + 255) // 256 * 256
+                assert one + tiled_rows * K.row_bytes(ty, cols) <= many <= one + tiled_rows * K.row_bytes(ty, cols) + 4 * 256
+    assert pkg.resident_bytes(pkg.Q4_K, 16, 100, 1) == 0      # not whole blocks
+    assert pkg.resident_bytes(3, 16, 256, 1) == 0             # Q4_1 is outside the eight dtypes
+    assert pkg.resident_bytes(pkg.Q8_0, 0, 32, 1) == 0
+    assert pkg.resident_bytes(pkg.Q8_0, 1 << 33, 32, 1) == 0  # rows beyond u32
+
+
 def test_cache_budget_env_grammar(lib):
     """langtax/src/native_gpu.rs:338-359: `auto` or decimal digits, nothing else."""
     is_auto, b = C.c_int(), C.c_size_t()

@@ -53,6 +53,22 @@ def test_topk_orders_descending_and_breaks_ties_towards_the_lower_index(llama):
             llama.topk([0.5, 0.3, 0.2], k)
 
 
+def test_topk_has_a_total_order_with_nans(llama):
+    """The reference's comparator calls a NaN a tie with everything (langtax/src/decode.rs:11369-11377), which orders
+    nothing once a NaN is present; here numbers come first, descending, then the NaNs, equal keys by index: the
+    result is defined for every input and is the reference's on every input without NaN."""
+    nan = float("nan")
+    assert llama.topk([nan, 0.3, 0.9, nan, 0.3], 5).tolist() == [2, 1, 4, 0, 3]
+    assert llama.topk([nan, nan, nan], 2).tolist() == [0, 1]
+    assert llama.topk([nan, -np.inf, nan], 1).tolist() == [1]
+    rng = np.random.default_rng(3)
+    for _ in range(50):   # many NaNs among many ties: same answer as a stable sort on (is NaN, -value)
+        v = rng.integers(0, 4, 64).astype(np.float32)
+        v[rng.random(64) < 0.3] = np.nan
+        key = np.where(np.isnan(v), np.inf, -v)
+        assert llama.topk(v, 64).tolist() == np.argsort(key, kind="stable").tolist()
+
+
 def test_router_weights_closed_forms(llama):
     # uniform probabilities: equal weights 1 / k
     w = llama.router_weights(np.full(8, 0.125, np.float32), [0, 1])

@@ -102,7 +102,7 @@ def test_every_extern_declaration_matches_the_header():
     # what the wrappers of gpu.rs and the reference's call sites need is bound
     for needed in ("lnh_create", "lnh_destroy", "lnh_memory_info", "lnh_upload_f32", "lnh_upload_packed", "lnh_matrix_free",
                    "lnh_gemv", "lnh_gemm", "lnh_gemm_grouped", "lnh_last_error", "lnh_thread_error", "lnq_gemm",
-                   "lnh_gemm_device_noalloc"):
+                   "lnh_gemm_device_noalloc", "lnh_matrix_info", "lnh_resident_bytes"):
         assert needed in r, needed
     # measurement and test helpers of the header are deliberately left out of the binding
     assert set(c) - set(r) <= {"lnh_calibration_copy", "lnh_calibration_read", "lnq_parse_cache_bytes", "lnq_automatic_cache_bytes",
@@ -147,6 +147,13 @@ def test_patch_names_only_the_wiring_files():
     assert any("upload_packed(ggml_type, rows, cols, packed)" in l for l in added)
     assert any('native-hip = ["dep:llama-native-hip", "llama-native-hip/hip"]' in l for l in added)
     assert any("LLAMA_HIP_CACHE_BYTES" in l for l in added)
+    # the residency charge is the C++ twin's (llama-rust_amd/csrc/residency.cpp: resident, recharge): what the matrix
+    # holds on the device plus the identity copy, asked from the library, and charged again after every product
+    # because the figure grows when the multi-token layout appears - never a constant multiple of the packed size
+    assert not any(re.search(r"checked_mul\(\s*\d+\s*\)", l) for l in added), "a constant multiple of the packed size"
+    assert any("resident_bytes(t, rows, cols, tokens)" in l for l in added)
+    assert any("device.checked_add(packed.len())" in l for l in added)
+    assert any(".device_bytes()" in l for l in added) and sum("recharge_last(state);" in l for l in added) == 2
     # hunk headers are consistent with their bodies (a hand-edited patch that no longer applies shows up here)
     for m in re.finditer(r"^@@ -(\d+),(\d+) \+(\d+),(\d+) @@.*\n((?:[ +\-].*\n|\n)*)", patch, flags=re.M):
         old_n, new_n, body = int(m.group(2)), int(m.group(4)), m.group(5).splitlines()

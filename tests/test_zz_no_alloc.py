@@ -51,7 +51,7 @@ def _both(gpu, hip, m, ty, rows, cols, tokens, w, rng):
     assert np.all(err <= 1e-4 * np.maximum(np.abs(exact), np.sqrt(np.mean(exact ** 2)) / 4))
 
 
-@pytest.mark.parametrize("ty", [K.Q4_K, K.Q4_0, K.Q6_K, K.Q8_0])
+@pytest.mark.parametrize("ty", [K.Q4_K, K.Q4_0, K.Q5_0, K.Q5_1, K.Q6_K, K.Q8_0])
 def test_noalloc_equals_gemm_device_twice_in_a_row(gpu, hip, ty):
     """A larger product, then a smaller one through the same static workspace (column shares, 16-token
     and 32-token tiles), each equal to lnh_gemm_device bit for bit and inside the oracle's bound."""
@@ -73,6 +73,64 @@ def test_noalloc_equals_gemm_device_twice_in_a_row(gpu, hip, ty):
     finally:
         m.close()
         m2.close()
+
+
+@pytest.mark.parametrize("ty", [K.F16, K.F32])
+def test_noalloc_plain_dtypes_with_shared_columns(gpu, hip, ty):
+    """F16 / F32 matrices with two or more tokens keep the partial sums of their column shares in the same static
+    array: few rows and many columns, so that the columns are shared between workgroups; then a smaller product."""
+    rng = np.random.default_rng(300 + ty)
+    rows, cols = 96, 14336
+    w = K.random_packed(ty, rows, cols, rng)
+    m = gpu.upload_packed(ty, rows, cols, w)
+    rows2, cols2 = 40, 4096
+    w2 = K.random_packed(ty, rows2, cols2, rng)
+    m2 = gpu.upload_packed(ty, rows2, cols2, w2)
+    try:
+        _both(gpu, hip, m, ty, rows, cols, 33, w, rng)
+        _both(gpu, hip, m2, ty, rows2, cols2, 4, w2, rng)
+        _both(gpu, hip, m, ty, rows, cols, 2, w, rng)
+    finally:
+        m.close()
+        m2.close()
+
+
+@pytest.mark.parametrize("ty,tokens", [(K.Q4_K, 24), (K.Q5_1, 7), (K.Q8_0, 70), (K.F16, 5)])
+def test_noalloc_recorded_into_a_graph_and_replayed(gpu, hip, ty, tokens):
+    """What the entry point is for: a call recorded while the stream is being captured (nothing may be allocated
+    there), replayed several times with the program's own eager work and synchronisations between the replays, the
+    input changed between replays; every replay equal bit for bit to lnh_gemm_device on the same input."""
+    rng = np.random.default_rng(500 + ty)
+    rows, cols = 640, 4096
+    w = K.random_packed(ty, rows, cols, rng, signed=False, scale=0.02)
+    m = gpu.upload_packed(ty, rows, cols, w)
+    stream = hip.Stream()
+    xd = hip.DeviceBuffer(tokens * cols * 4)
+    ya, yb = hip.DeviceBuffer(tokens * rows * 4), hip.DeviceBuffer(tokens * rows * 4)
+    graph = None
+    try:
+        gpu.prepare(m, tokens)   # before the capture: the capture itself may not allocate
+        graph = hip.Graph(stream, lambda s: gpu.gemm_device_noalloc(m, tokens, xd.ptr, ya.ptr, s.ptr))
+        for replay in range(3):
+            x = rng.normal(0, 1, tokens * cols).astype(np.float32)
+            xd.upload(x)
+            ya.fill_byte(0xff)
+            yb.fill_byte(0xff)
+            hip.device_synchronize()
+            graph.launch()
+            stream.synchronize()
+            gpu.gemm_device(m, tokens, xd.ptr, yb.ptr)   # eager work of the program between the replays
+            gpu.synchronize()
+            a, b = ya.to_numpy(np.float32), yb.to_numpy(np.float32)
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), f"replay {replay}"
+            exact, mag = O.gemm_f64_mag(ty, cols, tokens, w, x, rows)
+            assert np.all(np.abs(a.reshape(tokens, rows) - exact) <= K.single_kernel_bound(cols, mag)), f"replay {replay}"
+    finally:
+        if graph is not None:
+            graph.destroy()
+        for buf in (xd, ya, yb):
+            buf.free()
+        m.close()
 
 
 def test_noalloc_rejects_what_does_not_fit(gpu, hip, pkg):
