@@ -15,9 +15,13 @@
 //   Q6_K : ql[nb][128] | qh[nb][64] | sc[nb][16] int8 | d[nb] f16
 //   F16 / F32 : the row itself, zero-padded to a multiple of 8 elements
 //
-// Nothing is expanded: the planes hold exactly the bytes of the GGUF blocks
+// Nothing is expanded: the planes hold exactly the bits of the GGUF blocks
 // (F16/F32 rows gain at most 7 elements of zero padding) and every code plane
-// row starts 16-byte aligned.
+// row starts 16-byte aligned.  One field is permuted inside its 32 bits: the
+// fifth bits qh of a Q5 block are stored so that the four bits a code dword
+// needs sit at the same bit of its four bytes (repack.inc, q5_permuted), and
+// Q5_0's planes hold the complement of that word (its kernel wants the bit
+// flipped).
 //
 // Code planes are stored piece-major.  The single-token kernels give one lane a
 // "unit" of a row (a 256-column super-block; 8 consecutive blocks of Q4_0/Q5_x;
