@@ -668,11 +668,12 @@ struct FgPlan {
     size_t part_bytes;
 };
 static void fg_plan(const MatView &m, uint32_t tokens, FgPlan &p) {
-    p.tt = tokens > 32 ? 2 : 1;
-    const uint32_t tile_tok = 32u * (uint32_t)p.tt;
+    p.tt = tokens > 32 ? 2 : tokens > 16 ? 1 : 0;   // 0: a 16-token tile
+    const uint32_t tile_tok = p.tt == 0 ? 16u : 32u * (uint32_t)p.tt;
     const uint32_t tok_tiles = (tokens + tile_tok - 1) / tile_tok, row_tiles = (m.rows + FG_ROWS - 1) / FG_ROWS;
     const uint32_t tiles = tok_tiles * row_tiles, n_steps = (m.cols + FG_K - 1) / FG_K;
-    uint32_t ks = (uint32_t)(2 * g_cu_count) / (tiles ? tiles : 1);   // about two workgroups per CU
+    // about two workgroups per CU (16-token tiles measured at 1 / 2 / 3 / 4 per CU: F16 4096x14336, 8 tokens, 51 / 40 / 40 / 44 us)
+    uint32_t ks = (uint32_t)(2 * g_cu_count) / (tiles ? tiles : 1);
     if (ks > n_steps / 8) ks = n_steps / 8;                           // a share is at least 256 columns
     if (ks > 32) ks = 32;
     if (ks < 1) ks = 1;
@@ -690,7 +691,7 @@ static void fg_plan(const MatView &m, uint32_t tokens, FgPlan &p) {
 
 template <uint32_t T, int TT>
 static hipError_t launch_fg_main(hipStream_t stream, const FgPlan &p) {
-    constexpr size_t lds = (size_t)2 * (FG_ROWS + 32 * TT) * FG_LD * sizeof(float);
+    constexpr size_t lds = (size_t)2 * (FG_ROWS + (TT == 0 ? 16 : 32 * TT)) * FG_LD * sizeof(float);
     auto kern = gemm_fmfma_kernel<T, TT>;
     static bool configured = false;
     if (lds > 48 * 1024 && !configured) {
@@ -711,8 +712,10 @@ static hipError_t launch_fg(hipStream_t stream, const MatView &m, uint32_t token
     p.job.y = y;
     p.job.part = static_cast<float *>(ws);
     hipError_t e;
-    if (m.type == T_F16) e = p.tt == 2 ? launch_fg_main<T_F16, 2>(stream, p) : launch_fg_main<T_F16, 1>(stream, p);
-    else e = p.tt == 2 ? launch_fg_main<T_F32, 2>(stream, p) : launch_fg_main<T_F32, 1>(stream, p);
+    if (m.type == T_F16)
+        e = p.tt == 2 ? launch_fg_main<T_F16, 2>(stream, p) : p.tt == 1 ? launch_fg_main<T_F16, 1>(stream, p) : launch_fg_main<T_F16, 0>(stream, p);
+    else
+        e = p.tt == 2 ? launch_fg_main<T_F32, 2>(stream, p) : p.tt == 1 ? launch_fg_main<T_F32, 1>(stream, p) : launch_fg_main<T_F32, 0>(stream, p);
     if (e != hipSuccess || p.job.ksplit < 2) return e;
     const size_t total = (size_t)tokens * m.rows, vec = (total + 3) / 4, blocks = (vec + 255) / 256;
     hipLaunchKernelGGL(fg_reduce_kernel, dim3((unsigned)(blocks < 512 ? blocks : 512)), dim3(256), 0, stream, p.job.part, y, total,
