@@ -606,7 +606,16 @@ def main():
         if head:
             gpu.calibration_read(at, head_bytes // 16 * 16, s.ptr)
 
+    def enqueue_read_layers_merged(s=stream):
+        """The same bytes with one read launch per layer instead of four: what the kernel boundaries inside a layer
+        cost a reader, i.e. the most a kernel spanning a layer's products could gain on them."""
+        at, per_layer = read_buf.ptr, sum(read_sizes)
+        for _ in range(args.layers):
+            gpu.calibration_read(at, per_layer, s.ptr)
+            at += per_layer
+
     enqueue_read_step(); stream.synchronize()
+    enqueue_read_layers_merged(); stream.synchronize()
 
     if not args.no_graph:
         graphs = {"step": hip.Graph(stream, enqueue_step), "layers": hip.Graph(stream, enqueue_layers),
@@ -614,6 +623,7 @@ def main():
         for label, b in shape_batches.items():
             graphs[label] = hip.Graph(stream, lambda s, b=b: gpu.gemm_batch_device(b, s.ptr))
         graphs["read layers"] = hip.Graph(stream, lambda s: enqueue_read_step(s, head=False))
+        graphs["read layers merged"] = hip.Graph(stream, enqueue_read_layers_merged)
         for k, label in enumerate(shape_groups):
             graphs["read " + label] = hip.Graph(stream, lambda s, k=k: enqueue_read_step(s, without=k, head=False))
         run = {k: g.launch for k, g in graphs.items()}
@@ -622,6 +632,7 @@ def main():
         for label, b in shape_batches.items():
             run[label] = lambda b=b: gpu.gemm_batch_device(b, stream.ptr)
         run["read layers"] = lambda: enqueue_read_step(stream, head=False)
+        run["read layers merged"] = lambda: enqueue_read_layers_merged(stream)
         for k, label in enumerate(shape_groups):
             run["read " + label] = lambda k=k: enqueue_read_step(stream, without=k, head=False)
 
@@ -695,6 +706,7 @@ def main():
                             "achieved": round(shape_bytes[label] / us / 1e3, 1), "frac": round(shape_bytes[label] / us / 1e3 / HBM_PEAK_GBS, 4),
                             "plain_read_us": round(read_us, 2), "frac_of_plain_read": round(read_us / us, 3)}
     read_step_us = replay_us("read_step", max(3, args.steps // 2))
+    read_merged_us = replay_us("read layers merged", reps)
     traffic = profiled_traffic()
 
     out = {
@@ -722,7 +734,11 @@ def main():
                          "what": "a kernel that only reads, launched as the same chain at the same byte counts (4 per layer + head)",
                          "step_us": round(read_step_us, 1), "gbs": round(step_bytes / read_step_us / 1e3, 1),
                          "frac_of_peak": round(step_bytes / read_step_us / 1e3 / HBM_PEAK_GBS, 4),
-                         "this_step_vs_plain_read": round(read_step_us / (ms_per_step * 1e3), 3)}},
+                         "this_step_vs_plain_read": round(read_step_us / (ms_per_step * 1e3), 3),
+                         "layer_us_four_launches": round(read_layers_us / args.layers, 2),
+                         "layer_us_one_launch": round(read_merged_us / args.layers, 2),
+                         "layer_note": "a layer's 122.9 MB read by four dependent launches (the products' sizes) and by one: "
+                                       "the difference is what the three kernel boundaries inside a layer cost a reader"}},
         "other_kernels": {"gemv_q6k_kernel (head)": {"achieved": round(head_gbs, 1), "unit": "GB/s",
                                                      "frac": round(head_gbs / HBM_PEAK_GBS, 4),
                                                      "launch_us": round(head_ms * 1e3, 2)}},
