@@ -361,6 +361,7 @@ def other_workloads(pkg, hip, gpu, stream, rng, cpu):
     us_b = timed_us(hip, stream, layer_batched, sets, 5)
     for buf, _ in refs.values():
         buf.fill_byte(0xff)   # NaN patterns: a job that wrote to the wrong place leaves them standing
+    hip.device_synchronize()  # the fill runs on the null stream, which the (non-blocking) launch stream does not wait for
     layer_batched(0); stream.synchronize()
     for name, (buf, ref) in refs.items():
         if not np.allclose(buf.to_numpy(np.float32), ref, rtol=1e-4, atol=1e-4 * float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))):

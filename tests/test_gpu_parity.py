@@ -37,23 +37,45 @@ def gpu(pkg):
     g.close()
 
 
-# (case, outputs, max |a-e| / bound, max relative error away from zero, outputs near zero, max error in u of sum|wx|,
-#  then the last-but-two and the last figure again for the restated AVX2 CPU kernels on the same inputs)
+# One entry per named case: (case, outputs, max |a-e| / bound, max relative error away from zero, outputs near zero,
+#  max error in u of sum|wx|, the last-but-two and the last figure again for the restated AVX2 CPU kernels on the same
+#  inputs, max |a-e| over what tier (iii) allows).
 REPORT = []
+
+
+def _report_lines(entries):
+    """The figures behind the tolerance tiers: one line per named case, then one per benchmark configuration (worst
+    over its cases).  `literal` is the benchmark's own criterion read literally - max |a-e|/|e| over the outputs
+    with |e| >= 1e-3 rms(e), against 1e-4 - for the GPU and for the reference's AVX2 order on the same inputs;
+    `tier iii` is max |a-e| / (1e-4 max(|e|, rms(e)/4)), the criterion the tests assert (<= 1)."""
+    head = ("case | outputs | max |a-e| / gamma(n+3) sum|wx| | literal: max |a-e|/|e| where |e| >= 1e-3 rms(e) (1e-4 asked) | "
+            "outputs below that | tier iii: max |a-e| / (1e-4 max(|e|, rms/4)) | max |a-e| in u = 2^-24 of sum|wx| | "
+            "CPU (AVX2 order) literal | CPU: max |a-e| in u")
+    lines = [head]
+    per_config = {}
+    for name, n, r_bound, r_rel, n_small, r_u, c_rel, c_u, r_iii in entries:
+        lines.append(f"{name} | {n} | {r_bound:.4f} | {r_rel:.3e} | {n_small} | {r_iii:.3f} | {r_u:.2f} | {c_rel:.3e} | {c_u:.2f}")
+        key = " ".join(name.split()[:2])
+        a = per_config.setdefault(key, [0, 0.0, 0.0, 0, 0.0, 0.0, 0.0, 0.0])
+        a[0] += n
+        a[3] += n_small
+        for i, v in ((1, r_bound), (2, r_rel), (4, r_iii), (5, r_u), (6, c_rel), (7, c_u)):
+            a[i] = max(a[i], v)
+    lines.append("")
+    lines.append("per configuration (worst over its cases):")
+    for key, (n, r_bound, r_rel, n_small, r_iii, r_u, c_rel, c_u) in per_config.items():
+        lines.append(f"{key} | {n} | {r_bound:.4f} | {r_rel:.3e} ({'meets' if r_rel <= 1e-4 else 'exceeds'} 1e-4) | {n_small} | "
+                     f"{r_iii:.3f} | {r_u:.2f} | {c_rel:.3e} ({'meets' if c_rel <= 1e-4 else 'exceeds'} 1e-4) | {c_u:.2f}")
+    return lines
 
 
 @pytest.fixture(scope="module", autouse=True)
 def parity_report():
-    """After the module's tests: the figures behind the three tolerance tiers, one line per named case,
-    printed and (when PARITY_REPORT names a file) written out."""
+    """After the module's tests: the report of _report_lines, printed and (when PARITY_REPORT names a file) written out."""
     yield
     if not REPORT:
         return
-    lines = ["case | outputs | max |a-e| / gamma(n+3) sum|wx| | max |a-e|/|e| where |e| >= 1e-3 rms(e) | outputs below that | "
-             "max |a-e| in u = 2^-24 of sum|wx| | CPU (AVX2 order): max |a-e|/|e| | CPU: max |a-e| in u"]
-    for name, n, r_bound, r_rel, n_small, r_u, c_rel, c_u in REPORT:
-        lines.append(f"{name} | {n} | {r_bound:.4f} | {r_rel:.3e} | {n_small} | {r_u:.2f} | {c_rel:.3e} | {c_u:.2f}")
-    text = "\n".join(lines)
+    text = "\n".join(_report_lines(REPORT))
     print("\n" + text)
     path = os.environ.get("PARITY_REPORT")
     if path:
@@ -90,7 +112,8 @@ def check(actual, ty, n_cols, n_tokens, n_rows, w, x, name="", strict=False):
                        float(np.max(err[away] / np.abs(exact[away]))) if away.any() else 0.0, int(err.size - away.sum()),
                        float(np.max(err / np.maximum(mag, 1e-300)) / K.U),
                        float(np.max(cerr[away] / np.abs(exact[away]))) if away.any() else 0.0,
-                       float(np.max(cerr / np.maximum(mag, 1e-300)) / K.U)))
+                       float(np.max(cerr / np.maximum(mag, 1e-300)) / K.U),
+                       float(np.max(err / np.maximum(allowed, 1e-300)))))
     return err, mag
 
 
