@@ -1077,7 +1077,7 @@ __global__ __launch_bounds__(256) void read_kernel(const uint4 *__restrict__ p, 
 #pragma unroll
     for (int k = 0; k < 8; k++) {
         const size_t i = base + (size_t)k * 256;
-        v[k] = p[i < n16 ? i : 0];
+        v[k] = stream_load16(reinterpret_cast<const uint8_t *>(p + (i < n16 ? i : 0)));  // read once: the products' own kind of load
     }
     uint32_t a = 0;
 #pragma unroll
