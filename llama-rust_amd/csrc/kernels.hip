@@ -595,11 +595,13 @@ static hipError_t launch_mm16_main(hipStream_t stream, const MmBatch &b) {
     return hipGetLastError();
 }
 
-// Workgroups per job of the share reduction: one float4 per thread where that fills fewer than 512.
+// Workgroups per job of the share reduction: one float4 per thread (one float for small jobs, as the kernel
+// chooses) where that fills fewer than 512.
 static uint32_t mm_reduce_blocks(const MmBatch &b) {
     size_t most = 1;
     for (uint32_t j = 0; j < b.n_jobs; j++) {
-        const size_t vec = ((size_t)b.job[j].tokens * b.job[j].m.rows + 3) / 4, blocks = (vec + 255) / 256;
+        const size_t total = (size_t)b.job[j].tokens * b.job[j].m.rows;
+        const size_t per_thread = total >= MM_REDUCE_WIDE_MIN ? 4 : 1, blocks = ((total + per_thread - 1) / per_thread + 255) / 256;
         if (b.job[j].ksplit > 1 && blocks > most) most = blocks;
     }
     return (uint32_t)(most < 512 ? most : 512);
